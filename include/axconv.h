@@ -1,0 +1,158 @@
+/*
+ * axconv -- C ABI of the MI355X (gfx950) implementation of TFApprox's
+ * ApproxConv2DWithMinMaxVars hot path.
+ *
+ * Plain C: opaque handles, raw device pointers, sizes, int status codes.  No C++ or
+ * framework types cross this boundary.  All tensor pointers are DEVICE pointers
+ * (hipMalloc'd or owned by any framework that hands out HIP device memory); the four
+ * min/max values are host scalars passed by value, as the reference pins them to host
+ * memory (tf2/src/approx_nn_conv_ops.cpp:691-694).  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  Launch calls are asynchronous on that stream, allocate
+ * nothing and keep no state between calls: the caller owns the workspace.
+ *
+ * Each declaration cites the reference interface (paths under tf2/src/) it replaces.
+ */
+#ifndef AXCONV_H
+#define AXCONV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes; the reference reports the same conditions through tensorflow::Status
+ * (errors::InvalidArgument / errors::Unimplemented, approx_nn_conv_ops.cpp:120,162,224,231,287-303). */
+enum {
+    AXC_OK = 0,
+    AXC_INVALID_ARGUMENT = 1,
+    AXC_UNIMPLEMENTED = 2,
+    AXC_RUNTIME_ERROR = 3 /* a HIP call failed; the reference ignores CUDA return codes */
+};
+
+enum { AXC_PAD_VALID = 0, AXC_PAD_SAME = 1, AXC_PAD_EXPLICIT = 2 };
+enum { AXC_FORMAT_NHWC = 0, AXC_FORMAT_NCHW = 1 };
+
+/* Attributes and shapes of one op invocation: the op's attrs (approx_nn_ops.cpp:46-53,
+ * parsed at approx_nn_conv_ops.cpp:254-309) plus the input/filter shapes read in Compute
+ * (approx_nn_conv_ops.cpp:311-404).  strides/dilations are given in the data_format's own
+ * order, four entries each, exactly as the attrs hold them. */
+typedef struct axc_conv2d_desc {
+    int64_t input_shape[4];   /* in data_format order (NHWC: N,H,W,C) */
+    int64_t filter_shape[4];  /* HWIO: rows, cols, in_depth, out_depth */
+    int32_t strides[4];
+    int32_t dilations[4];
+    int32_t padding;          /* AXC_PAD_* */
+    int32_t data_format;      /* AXC_FORMAT_* */
+    int32_t num_bits;         /* only 8 is supported (approx_ops_types.h:218) */
+    int64_t explicit_paddings[8];
+} axc_conv2d_desc;
+
+/* Mirrors tensorflow::ApproxConv2DDimensions (approx_nn_conv_ops.h:56-79). */
+typedef struct axc_conv2d_dims {
+    int32_t batch, input_rows, input_cols, in_depth;
+    int32_t filter_rows, filter_cols, patch_depth, out_depth;
+    int32_t stride_rows, stride_cols, dilation_rows, dilation_cols;
+    int64_t out_rows, out_cols;
+    int64_t pad_rows_before, pad_rows_after, pad_cols_before, pad_cols_after;
+} axc_conv2d_dims;
+
+/* Mirrors BaseTableApproxOpType_t::OpQuantProps_t (approx_ops_types.h:79-97). */
+typedef struct axc_quant_props {
+    float input_scale, input_inv_scale, input_offset;
+    float filter_scale, filter_inv_scale, filter_offset;
+    float s1xs2, m1, m2, m1xm2;
+    int32_t input_zero_code; /* code of the value 0.0f: what padding taps look up */
+} axc_quant_props;
+
+/* Device-resident truth table.  Immutable after creation; may be shared by concurrent calls. */
+typedef struct axc_table axc_table;
+
+const char *axc_status_string(int status);
+/* Message of the last failing call on this thread (the reference's error text where it has one). */
+const char *axc_last_error(void);
+
+/* Replaces the GPU table upload, TableApproxOpType_t<GpuDevice> ctor (cuda/approx_ops_types.cu:20-42):
+ * host_table is uint16[65536], index (input_code << 8) | filter_code (approx_nn_conv_kernels.cpp:245). */
+int axc_table_create(const uint16_t *host_table, axc_table **out);
+/* Replaces BaseTableApproxOpType_t ctor + LoadLookupTable (approx_ops_types.h:99-122,205-216):
+ * empty or NULL filename -> exact products; short read -> AXC_INVALID_ARGUMENT
+ * "ApproxTF: Couldn't read the lookup table!"; num_bits != 8 -> AXC_INVALID_ARGUMENT. */
+int axc_table_create_from_file(const char *filename, int num_bits, axc_table **out);
+/* Replaces ~TableApproxOpType_t<GpuDevice> (cuda/approx_ops_types.cu:44-49). */
+int axc_table_destroy(axc_table *table);
+
+/* Replaces BaseTableApproxOpType_t::Update / UpdateVarQuantProps / Nudge
+ * (approx_ops_types.h:29-49,135-197), stateless. */
+int axc_quant_props_compute(float input_min, float input_max, float filter_min, float filter_max,
+                            axc_quant_props *out);
+
+/* Replaces InitApproxConv2DParameters + ComputeApproxConv2DDimensions
+ * (approx_nn_conv_ops.cpp:254-404), including their argument checks. */
+int axc_conv2d_geometry(const axc_conv2d_desc *desc, axc_conv2d_dims *dims);
+
+/* Scratch the launch calls below need for this desc (replaces the three allocate_temp calls at
+ * approx_nn_conv_ops.cpp:590-613). */
+int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
+int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
+
+/* The op: replaces ApproxConv2DOp::Compute -> LaunchApproxConv2DOp<GPUDevice> and the kernels it
+ * launches (approx_nn_conv_ops.cpp:420-460,510-664; cuda/approx_nn_conv_kernels.cu:296-627).
+ * input: float NHWC, filter: float HWIO, output: float NHWC [N,out_rows,out_cols,out_depth]. */
+int axc_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc,
+                      const float *input, const float *filter,
+                      float input_min, float input_max, float filter_min, float filter_max,
+                      float *output, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Depthwise variant (filter [rows, cols, C, 1]).  The reference has none: its CPU launcher rejects
+ * in_depth != filter in_depth (approx_nn_conv_ops.cpp:229-232).  Defined as the dense op applied to
+ * every channel on its own with the tensor-wide min/max. */
+int axc_depthwise_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc,
+                                const float *input, const float *filter,
+                                float input_min, float input_max, float filter_min, float filter_max,
+                                float *output, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- parity entry points (stages of the op, exposed so each can be checked bit for bit) ---- */
+
+/* The quantize expression (approx_nn_conv_kernels.cpp:193,197,243,293) on n floats:
+ * codes[i] = uint8((v[i] - offset) * inv_scale + 0.5f), offset/inv_scale from (min, max). */
+int axc_quantize(const float *values, int64_t n, float min, float max, uint8_t *codes, void *stream);
+
+/* Same as axc_conv2d_minmax / axc_depthwise_conv2d_minmax but stores the int32 sums of table
+ * entries (the `total` of approx_nn_conv_kernels.cpp:235-247 before the epilogue) instead of floats. */
+int axc_conv2d_minmax_acc_i32(const axc_table *table, const axc_conv2d_desc *desc,
+                              const float *input, const float *filter,
+                              float input_min, float input_max, float filter_min, float filter_max,
+                              int32_t *acc, void *workspace, size_t workspace_bytes, void *stream);
+int axc_depthwise_conv2d_minmax_acc_i32(const axc_table *table, const axc_conv2d_desc *desc,
+                                        const float *input, const float *filter,
+                                        float input_min, float input_max, float filter_min, float filter_max,
+                                        int32_t *acc, void *workspace, size_t workspace_bytes, void *stream);
+
+/* LUT-GEMM on caller-supplied codes: input_codes uint8 NHWC, filter_codes uint8 HWIO,
+ * input_zero_code is what out-of-bounds taps look up.  acc: int32 [N,out_rows,out_cols,out_depth]. */
+int axc_conv2d_codes_acc_i32(const axc_table *table, const axc_conv2d_desc *desc,
+                             const uint8_t *input_codes, const uint8_t *filter_codes, int input_zero_code,
+                             int32_t *acc, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- measurement -------------------------------------------------------------------------- */
+
+/* Per-kernel timing with HIP events recorded on the launch stream.  While enabled, every kernel the
+ * launch calls enqueue is bracketed by two events; axc_profile_read synchronizes them and returns the
+ * accumulated milliseconds and launch count per kernel name since the last reset. */
+int axc_profile_enable(int enable);
+int axc_profile_reset(void);
+int axc_profile_read(int index, char *name, size_t name_bytes, double *total_ms, int64_t *launches);
+
+/* Conflict-free ds_read_u16 gather rate of this GPU (lookups per second over all CUs): the measured
+ * ceiling of the LDS-lookup roofline. */
+int axc_lds_gather_peak(double *lookups_per_second, void *stream);
+
+/* Properties of the current device the planner uses. */
+int axc_device_info(int *compute_units, int *lds_bytes_per_workgroup, int *clock_khz);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXCONV_H */

@@ -1,0 +1,774 @@
+// C-ABI entry points of libaxconv_hip.so: validation, geometry, planning, workspace carving, launches.
+#include "axconv_internal.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+using namespace axc;
+
+struct axc_table {
+    uint16_t *dev_tableT; // [256 filter code][256 input code]
+    int device;
+};
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int status, const char *msg)
+{
+    g_last_error = msg;
+    return status;
+}
+
+int fail_hip(hipError_t e, const char *what)
+{
+    g_last_error = std::string(what) + ": " + hipGetErrorString(e);
+    return AXC_RUNTIME_ERROR;
+}
+
+#define AXC_HIP(call)                                \
+    do {                                             \
+        hipError_t e_ = (call);                      \
+        if (e_ != hipSuccess)                        \
+            return fail_hip(e_, #call);              \
+    } while (0)
+
+// ---- profiling: events around each kernel, on the launch stream ----
+struct ProfEntry {
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> pending;
+    double total_ms = 0.0;
+    int64_t launches = 0;
+};
+std::mutex g_prof_mutex;
+bool g_prof_enabled = false;
+std::map<std::string, ProfEntry> g_prof;
+
+struct ProfScope {
+    const char *name;
+    hipStream_t stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    bool on;
+    ProfScope(const char *n, hipStream_t s) : name(n), stream(s), on(g_prof_enabled)
+    {
+        if (on && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess)
+            (void)hipEventRecord(e0, stream);
+        else
+            on = false;
+    }
+    ~ProfScope()
+    {
+        if (!on)
+            return;
+        (void)hipEventRecord(e1, stream);
+        std::lock_guard<std::mutex> lock(g_prof_mutex);
+        g_prof[name].pending.emplace_back(e0, e1);
+    }
+};
+
+void prof_drain_locked(ProfEntry &pe)
+{
+    for (auto &ev : pe.pending) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(ev.second) == hipSuccess && hipEventElapsedTime(&ms, ev.first, ev.second) == hipSuccess) {
+            pe.total_ms += ms;
+            pe.launches += 1;
+        }
+        (void)hipEventDestroy(ev.first);
+        (void)hipEventDestroy(ev.second);
+    }
+    pe.pending.clear();
+}
+
+// ---- quantization parameters (approx_ops_types.h:29-49,135-197) ----
+// Every float operation rounds on its own (volatile), as in the reference build.
+void nudge(float min, float max, float *nudged_min, float *nudged_max, float *scale, int *zero_point)
+{
+    const float qmin = 0.0f, qmax = 255.0f;
+    volatile float range = max - min;
+    volatile float sc = range / (qmax - qmin);
+    volatile float ratio = min / sc;
+    volatile float zp_from_min = qmin - ratio;
+    int zp;
+    if (zp_from_min < qmin)
+        zp = 0;
+    else if (zp_from_min > qmax)
+        zp = 255;
+    else
+        zp = (int)(uint16_t)roundf(zp_from_min);
+    volatile float lo = (qmin - (float)zp) * sc;
+    volatile float hi = (qmax - (float)zp) * sc;
+    *nudged_min = lo;
+    *nudged_max = hi;
+    *scale = sc;
+    *zero_point = zp;
+}
+
+void var_quant_props(float min, float max, float *scale, float *inv_scale, float *offset)
+{
+    float s = 0.0f, inv = 0.0f, nmin = 0.0f, nmax = 0.0f;
+    int zp = 0;
+    if (min != 0.0f || max != 0.0f) {
+        nudge(min, max, &nmin, &nmax, &s, &zp);
+        volatile float i = 1.0f / s;
+        inv = i;
+    }
+    *scale = s;
+    *inv_scale = inv;
+    *offset = nmin;
+}
+
+int host_quantize(float v, float offset, float inv_scale)
+{
+    volatile float d = v - offset;
+    volatile float pr = d * inv_scale;
+    volatile float t = pr + 0.5f;
+    float tt = t;
+    if (!(tt > 0.0f))
+        return 0;
+    if (tt >= 255.0f)
+        return 255;
+    return (int)tt;
+}
+
+// ---- geometry (approx_nn_conv_ops.cpp:254-404) ----
+int windowed_output_size(int64_t in, int64_t filter, int64_t dilation, int64_t stride, int padding,
+                         int64_t *out, int64_t *before, int64_t *after)
+{
+    const int64_t eff = (filter - 1) * dilation + 1;
+    if (padding == AXC_PAD_VALID) {
+        *out = (in - eff + stride) / stride;
+        *before = *after = 0;
+    } else if (padding == AXC_PAD_SAME) {
+        *out = (in + stride - 1) / stride;
+        int64_t needed = (*out - 1) * stride + eff - in;
+        if (needed < 0)
+            needed = 0;
+        *before = needed / 2;
+        *after = needed - *before;
+    } else {
+        *out = (in + *before + *after - eff + stride) / stride;
+    }
+    if (*out < 0)
+        return fail(AXC_INVALID_ARGUMENT, "Computed output size would be negative");
+    return AXC_OK;
+}
+
+int geometry(const axc_conv2d_desc *d, axc_conv2d_dims *o)
+{
+    if (!d || !o)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    if (d->data_format != AXC_FORMAT_NHWC && d->data_format != AXC_FORMAT_NCHW)
+        return fail(AXC_INVALID_ARGUMENT, "Invalid data format");
+    const bool nhwc = d->data_format == AXC_FORMAT_NHWC;
+    const int iN = 0, iC = nhwc ? 3 : 1, iH = nhwc ? 1 : 2, iW = nhwc ? 2 : 3;
+    if (d->strides[iN] != 1 || d->strides[iC] != 1)
+        return fail(AXC_INVALID_ARGUMENT,
+                    "Current implementation does not yet support strides in the batch and depth dimensions.");
+    if (d->strides[iH] <= 0 || d->strides[iW] <= 0)
+        return fail(AXC_INVALID_ARGUMENT, "Row and column strides should be larger than 0.");
+    if (d->dilations[iN] != 1 || d->dilations[iC] != 1)
+        return fail(AXC_INVALID_ARGUMENT,
+                    "Current implementation does not yet support dilations in the batch and depth dimensions.");
+    if (d->dilations[iH] <= 0 || d->dilations[iW] <= 0)
+        return fail(AXC_INVALID_ARGUMENT, "Dilated rates should be larger than 0.");
+    if (d->padding != AXC_PAD_VALID && d->padding != AXC_PAD_SAME && d->padding != AXC_PAD_EXPLICIT)
+        return fail(AXC_INVALID_ARGUMENT, "Invalid padding");
+    for (int i = 0; i < 4; ++i) {
+        if (d->input_shape[i] < 0 || d->input_shape[i] > INT32_MAX)
+            return fail(AXC_INVALID_ARGUMENT, "input is too large");
+        if (d->filter_shape[i] < 0 || d->filter_shape[i] > INT32_MAX)
+            return fail(AXC_INVALID_ARGUMENT, "filter is too large");
+    }
+    const int64_t in_depth = d->input_shape[iC], patch_depth = d->filter_shape[2];
+    if (patch_depth <= 0 || in_depth % patch_depth != 0)
+        return fail(AXC_INVALID_ARGUMENT, "input depth must be evenly divisible by filter depth");
+
+    o->batch = (int32_t)d->input_shape[iN];
+    o->input_rows = (int32_t)d->input_shape[iH];
+    o->input_cols = (int32_t)d->input_shape[iW];
+    o->in_depth = (int32_t)in_depth;
+    o->filter_rows = (int32_t)d->filter_shape[0];
+    o->filter_cols = (int32_t)d->filter_shape[1];
+    o->patch_depth = (int32_t)patch_depth;
+    o->out_depth = (int32_t)d->filter_shape[3];
+    o->stride_rows = d->strides[iH];
+    o->stride_cols = d->strides[iW];
+    o->dilation_rows = d->dilations[iH];
+    o->dilation_cols = d->dilations[iW];
+    o->pad_rows_before = o->pad_rows_after = o->pad_cols_before = o->pad_cols_after = 0;
+    if (d->padding == AXC_PAD_EXPLICIT) {
+        o->pad_rows_before = d->explicit_paddings[2 * iH];
+        o->pad_rows_after = d->explicit_paddings[2 * iH + 1];
+        o->pad_cols_before = d->explicit_paddings[2 * iW];
+        o->pad_cols_after = d->explicit_paddings[2 * iW + 1];
+    }
+    int rc = windowed_output_size(o->input_rows, o->filter_rows, o->dilation_rows, o->stride_rows, d->padding,
+                                  &o->out_rows, &o->pad_rows_before, &o->pad_rows_after);
+    if (rc != AXC_OK)
+        return rc;
+    return windowed_output_size(o->input_cols, o->filter_cols, o->dilation_cols, o->stride_cols, d->padding,
+                                &o->out_cols, &o->pad_cols_before, &o->pad_cols_after);
+}
+
+// Checks shared by every launch entry point; the reference's messages where it has them.
+int validate_for_launch(const axc_conv2d_desc *d, const axc_conv2d_dims &dm, bool depthwise)
+{
+    if (d->num_bits != 8)
+        return fail(AXC_INVALID_ARGUMENT, "only num_bits = 8 is supported");
+    if (d->data_format != AXC_FORMAT_NHWC)
+        return fail(AXC_UNIMPLEMENTED, "Generic conv implementation only supports NHWC tensor format for now.");
+    if (depthwise) {
+        if (d->filter_shape[3] != 1 || dm.patch_depth != dm.in_depth)
+            return fail(AXC_INVALID_ARGUMENT, "depthwise filter must be [rows, cols, in_depth, 1]");
+    } else if (dm.in_depth != dm.patch_depth) {
+        return fail(AXC_UNIMPLEMENTED, "Generic conv implementation does not support grouped convolutions for now.");
+    }
+    if (d->padding == AXC_PAD_EXPLICIT)
+        return fail(AXC_UNIMPLEMENTED, "Explicit padding is not implemented.");
+    const int64_t patch_len = (int64_t)dm.filter_rows * dm.filter_cols * dm.patch_depth;
+    if (patch_len > (int64_t)(16 * 1024 * 1024) / (int64_t)sizeof(float))
+        return fail(AXC_INVALID_ARGUMENT, "ApproxConv2DOp: Patch too large for buffer");
+    if (patch_len >= 32768) // 32768 * 65535 would overflow the int32 accumulator
+        return fail(AXC_INVALID_ARGUMENT, "patch length must be below 32768 for int32 accumulation");
+    if (dm.input_rows >= 32768 || dm.input_cols >= 32768 || dm.pad_rows_before >= 16384 ||
+        dm.pad_cols_before >= 16384)
+        return fail(AXC_INVALID_ARGUMENT, "image dimensions must be below 32768");
+    const int64_t out_elems = (int64_t)dm.batch * dm.out_rows * dm.out_cols * (depthwise ? dm.in_depth : dm.out_depth);
+    const int64_t in_elems = (int64_t)dm.batch * dm.input_rows * dm.input_cols * dm.in_depth;
+    if (out_elems >= ((int64_t)1 << 40) || in_elems >= ((int64_t)1 << 40))
+        return fail(AXC_INVALID_ARGUMENT, "tensor too large");
+    return AXC_OK;
+}
+
+ConvGeom make_geom(const axc_conv2d_dims &dm)
+{
+    ConvGeom g;
+    g.N = dm.batch; g.H = dm.input_rows; g.W = dm.input_cols; g.C = dm.in_depth;
+    g.KH = dm.filter_rows; g.KW = dm.filter_cols; g.Co = dm.out_depth;
+    g.OH = (int)dm.out_rows; g.OW = (int)dm.out_cols;
+    g.sh = dm.stride_rows; g.sw = dm.stride_cols; g.dh = dm.dilation_rows; g.dw = dm.dilation_cols;
+    g.ph = (int)dm.pad_rows_before; g.pw = (int)dm.pad_cols_before;
+    g.C4 = (g.C + 3) / 4;
+    g.M = (int64_t)g.N * g.OH * g.OW;
+    g.K = g.KH * g.KW * g.C;
+    return g;
+}
+
+int device_cus()
+{
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return 256;
+    return cus;
+}
+
+// Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
+// Derive cost per fill is constant; lookup cost per fill grows with the wavefront-rows a SIMD carries.
+DensePlan make_plan(const ConvGeom &g, int cus)
+{
+    DensePlan best{};
+    double best_cost = 1e300;
+    const int taps = g.KH * g.KW;
+    for (int nt : {16, 32, 64}) {
+        if (nt > 16 && nt / 2 >= g.Co)
+            continue; // half the columns of a wider tile would be padding
+        const int R = 64 / nt, ks = 64 / nt, subs = 4 / ks;
+        const int n_col = (g.Co + nt - 1) / nt;
+        const int fills = taps * g.C4 * subs;
+        const int64_t cap_wrows = (int64_t)kWaves * R; // wavefront-rows (64 pixels each) per tile
+        const int64_t total_wrows = (g.M + 63) / 64;
+        const int64_t min_tiles = (total_wrows + cap_wrows - 1) / cap_wrows;
+        // candidate row-tile counts: the minimum, and counts that fill whole rounds of CUs
+        std::vector<int64_t> cands{min_tiles};
+        for (int64_t rounds = 1; rounds <= 8; ++rounds) {
+            int64_t n_row = (rounds * cus) / n_col;
+            if (n_row > min_tiles && n_row <= total_wrows)
+                cands.push_back(n_row);
+            if (n_row + 1 > min_tiles && n_row + 1 <= total_wrows)
+                cands.push_back(n_row + 1);
+        }
+        if (total_wrows > min_tiles)
+            cands.push_back(total_wrows);
+        for (int64_t n_row : cands) {
+            const int64_t wrows = (total_wrows + n_row - 1) / n_row;  // per tile
+            const int64_t tiles = n_row * n_col;
+            const int64_t rounds = (tiles + cus - 1) / cus;
+            const double per_simd = (double)((wrows + 3) / 4);          // wavefront-rows on the busiest SIMD
+            const double per_fill = 450.0 + per_simd * (64.0 * 1.3 * 4.0); // cycles: derive + lookups
+            const double cost = (double)rounds * ((double)fills * per_fill + 3000.0);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best.nt = nt;
+                best.rows_per_tile = (int)(wrows * 64);
+                best.n_row_tiles = (int)((total_wrows + wrows - 1) / wrows);
+                best.n_col_tiles = n_col;
+                best.fills = fills;
+                best.grid = (int)((int64_t)best.n_row_tiles * n_col < cus ? (int64_t)best.n_row_tiles * n_col : cus);
+            }
+        }
+    }
+    return best;
+}
+
+inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct DenseWorkspace {
+    size_t xq_off, chsum_off, wq_off, fsum_off, total;
+};
+
+DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
+{
+    DenseWorkspace w;
+    size_t off = 0;
+    w.xq_off = off; off += align_up((size_t)g.N * g.H * g.C4 * g.W * 4);
+    w.chsum_off = off; off += align_up((size_t)g.N * g.H * g.W * 4);
+    w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
+    w.fsum_off = off; off += align_up((size_t)g.Co * 4);
+    w.total = off;
+    return w;
+}
+
+struct PreparedDense {
+    axc_conv2d_dims dims;
+    ConvGeom g;
+    DensePlan plan;
+    DenseWorkspace ws;
+    bool empty;
+};
+
+int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd)
+{
+    int rc = geometry(desc, &pd->dims);
+    if (rc != AXC_OK)
+        return rc;
+    rc = validate_for_launch(desc, pd->dims, false);
+    if (rc != AXC_OK)
+        return rc;
+    pd->g = make_geom(pd->dims);
+    pd->empty = pd->g.M * pd->g.Co == 0; // approx_nn_conv_ops.cpp:449
+    if (pd->empty || pd->g.K == 0) {
+        pd->plan = DensePlan{};
+        pd->ws = DenseWorkspace{};
+        return AXC_OK;
+    }
+    pd->plan = make_plan(pd->g, device_cus());
+    pd->ws = dense_workspace(pd->g, pd->plan);
+    return AXC_OK;
+}
+
+enum class DenseOut { Float, AccI32 };
+
+int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *input, const float *filter,
+              const uint8_t *input_codes, const uint8_t *filter_codes, int input_zero_code,
+              float in_min, float in_max, float f_min, float f_max, float *out_f, int32_t *out_i,
+              void *workspace, size_t workspace_bytes, void *stream_v)
+{
+    if (!table || !desc)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    PreparedDense pd;
+    int rc = prepare_dense(desc, &pd);
+    if (rc != AXC_OK)
+        return rc;
+    if (pd.empty)
+        return AXC_OK;
+    const bool codes_mode = input_codes != nullptr;
+    if ((!codes_mode && (!input || !filter)) || (codes_mode && !filter_codes) || (!out_f && !out_i))
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const ConvGeom &g = pd.g;
+
+    axc_quant_props qp;
+    memset(&qp, 0, sizeof(qp));
+    if (!codes_mode) {
+        axc_quant_props_compute(in_min, in_max, f_min, f_max, &qp);
+    } else {
+        if (input_zero_code < 0 || input_zero_code > 255)
+            return fail(AXC_INVALID_ARGUMENT, "input_zero_code must be in [0, 255]");
+        qp.input_zero_code = input_zero_code;
+    }
+
+    if (g.K == 0) { // no taps: every sum is empty
+        const int64_t n = g.M * g.Co;
+        if (out_i) {
+            AXC_HIP(hipMemsetAsync(out_i, 0, (size_t)n * 4, stream));
+        } else {
+            AXC_HIP(hipMemsetAsync(out_f, 0, (size_t)n * 4, stream));
+        }
+        return AXC_OK;
+    }
+    if (workspace_bytes < pd.ws.total || (!workspace && pd.ws.total))
+        return fail(AXC_INVALID_ARGUMENT, "workspace too small (see axc_conv2d_workspace_bytes)");
+    if (((uintptr_t)workspace & 255) != 0)
+        return fail(AXC_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+
+    char *ws = static_cast<char *>(workspace);
+    uint32_t *xq = reinterpret_cast<uint32_t *>(ws + pd.ws.xq_off);
+    float *chsum = reinterpret_cast<float *>(ws + pd.ws.chsum_off);
+    uint16_t *wq = reinterpret_cast<uint16_t *>(ws + pd.ws.wq_off);
+    float *fsum = reinterpret_cast<float *>(ws + pd.ws.fsum_off);
+
+    if (codes_mode) {
+        ProfScope ps("codes_relayout", stream);
+        AXC_HIP(launch_codes_relayout(input_codes, g, xq, stream));
+    } else {
+        ProfScope ps("quantize_relayout", stream);
+        AXC_HIP(launch_quantize_relayout(input, g, qp.input_offset, qp.input_inv_scale, xq,
+                                         out_f ? chsum : nullptr, stream));
+    }
+    {
+        ProfScope ps("filter_pack", stream);
+        AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, g, pd.plan, qp.filter_offset,
+                                   qp.filter_inv_scale, wq, (out_f && !codes_mode) ? fsum : nullptr, stream));
+    }
+
+    DenseParams p;
+    p.g = g;
+    p.plan = pd.plan;
+    p.xq = xq;
+    p.chsum = chsum;
+    p.wq = wq;
+    p.fsum = fsum;
+    p.tableT = table->dev_tableT;
+    p.out_f = out_f;
+    p.out_i = out_i;
+    p.s1xs2 = qp.s1xs2;
+    p.m1 = qp.m1;
+    p.m2 = qp.m2;
+    {
+        volatile float km = (float)g.K * qp.m1xm2;
+        p.k_m1xm2 = km;
+    }
+    const uint32_t zp = phys_row((uint32_t)qp.input_zero_code);
+    p.zp4 = zp * 0x01010101u;
+    {
+        ProfScope ps("lutgemm_expand", stream);
+        AXC_HIP(launch_dense(p, out_i != nullptr, stream));
+    }
+    return AXC_OK;
+}
+
+int run_depthwise(const axc_table *table, const axc_conv2d_desc *desc, const float *input, const float *filter,
+                  float in_min, float in_max, float f_min, float f_max, float *out_f, int32_t *out_i,
+                  void *workspace, size_t workspace_bytes, void *stream_v)
+{
+    if (!table || !desc)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    axc_conv2d_dims dm;
+    int rc = geometry(desc, &dm);
+    if (rc != AXC_OK)
+        return rc;
+    rc = validate_for_launch(desc, dm, true);
+    if (rc != AXC_OK)
+        return rc;
+    const int C = dm.in_depth, taps = dm.filter_rows * dm.filter_cols;
+    const int64_t M = (int64_t)dm.batch * dm.out_rows * dm.out_cols;
+    if (M * C == 0)
+        return AXC_OK;
+    if (!input || !filter || (!out_f && !out_i))
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    if (taps == 0) {
+        AXC_HIP(hipMemsetAsync(out_f ? (void *)out_f : (void *)out_i, 0, (size_t)M * C * 4, stream));
+        return AXC_OK;
+    }
+    const size_t wcodes_bytes = align_up((size_t)taps * C);
+    const size_t need = wcodes_bytes + align_up((size_t)C * 4);
+    if (workspace_bytes < need || !workspace)
+        return fail(AXC_INVALID_ARGUMENT, "workspace too small (see axc_depthwise_conv2d_workspace_bytes)");
+    if (((uintptr_t)workspace & 255) != 0)
+        return fail(AXC_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+    axc_quant_props qp;
+    axc_quant_props_compute(in_min, in_max, f_min, f_max, &qp);
+    uint8_t *wcodes = static_cast<uint8_t *>(workspace);
+    float *fsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + wcodes_bytes);
+    {
+        ProfScope ps("depthwise_filter", stream);
+        AXC_HIP(launch_depthwise_filter(filter, taps, C, qp.filter_offset, qp.filter_inv_scale, wcodes, fsum, stream));
+    }
+    DepthwiseParams p;
+    p.N = dm.batch; p.H = dm.input_rows; p.W = dm.input_cols; p.C = C;
+    p.KH = dm.filter_rows; p.KW = dm.filter_cols; p.OH = (int)dm.out_rows; p.OW = (int)dm.out_cols;
+    p.sh = dm.stride_rows; p.sw = dm.stride_cols; p.dh = dm.dilation_rows; p.dw = dm.dilation_cols;
+    p.ph = (int)dm.pad_rows_before; p.pw = (int)dm.pad_cols_before;
+    p.M = M;
+    p.x = input; p.wcodes = wcodes; p.fsum = fsum; p.tableT = table->dev_tableT;
+    p.out_f = out_f; p.out_i = out_i;
+    p.in_offset = qp.input_offset; p.in_inv_scale = qp.input_inv_scale;
+    p.s1xs2 = qp.s1xs2; p.m1 = qp.m1; p.m2 = qp.m2;
+    {
+        volatile float km = (float)taps * qp.m1xm2;
+        p.k_m1xm2 = km;
+    }
+    const int cus = device_cus();
+    const int64_t blocks_needed = (M * C + kBlockThreads - 1) / kBlockThreads;
+    const int grid = (int)(blocks_needed < cus ? blocks_needed : cus);
+    {
+        ProfScope ps("depthwise_lut", stream);
+        AXC_HIP(launch_depthwise(p, out_i != nullptr, grid, stream));
+    }
+    return AXC_OK;
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------------------------
+
+extern "C" {
+
+const char *axc_status_string(int status)
+{
+    switch (status) {
+    case AXC_OK: return "OK";
+    case AXC_INVALID_ARGUMENT: return "INVALID_ARGUMENT";
+    case AXC_UNIMPLEMENTED: return "UNIMPLEMENTED";
+    case AXC_RUNTIME_ERROR: return "RUNTIME_ERROR";
+    default: return "UNKNOWN";
+    }
+}
+
+const char *axc_last_error(void) { return g_last_error.c_str(); }
+
+int axc_table_create(const uint16_t *host_table, axc_table **out)
+{
+    if (!host_table || !out)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    // transpose to weight-code major: tableT[b][a] = T[(a << 8) | b]
+    std::vector<uint16_t> t(65536);
+    for (int a = 0; a < 256; ++a)
+        for (int b = 0; b < 256; ++b)
+            t[(size_t)b * 256 + a] = host_table[(size_t)a * 256 + b];
+    axc_table *tab = new axc_table;
+    tab->dev_tableT = nullptr;
+    hipError_t e = hipGetDevice(&tab->device);
+    if (e == hipSuccess)
+        e = hipMalloc(reinterpret_cast<void **>(&tab->dev_tableT), kTableBytes);
+    if (e == hipSuccess)
+        e = hipMemcpy(tab->dev_tableT, t.data(), kTableBytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (tab->dev_tableT)
+            (void)hipFree(tab->dev_tableT);
+        delete tab;
+        return fail_hip(e, "table upload");
+    }
+    *out = tab;
+    return AXC_OK;
+}
+
+int axc_table_create_from_file(const char *filename, int num_bits, axc_table **out)
+{
+    if (!out)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    if (num_bits != 8)
+        return fail(AXC_INVALID_ARGUMENT, "only num_bits = 8 is supported");
+    std::vector<uint16_t> t(65536, 0);
+    if (!filename || !filename[0]) {
+        for (uint32_t i = 0; i < 65536u; ++i)
+            t[i] = (uint16_t)((i >> 8) * (i & 0xFFu));
+    } else {
+        FILE *f = fopen(filename, "rb");
+        if (!f)
+            return fail(AXC_INVALID_ARGUMENT, "ApproxTF: Couldn't read the lookup table!");
+        std::vector<unsigned char> raw(kTableBytes);
+        const size_t got = fread(raw.data(), 1, kTableBytes, f);
+        fclose(f);
+        if (got != (size_t)kTableBytes)
+            return fail(AXC_INVALID_ARGUMENT, "ApproxTF: Couldn't read the lookup table!");
+        for (int i = 0; i < 65536; ++i)
+            t[i] = (uint16_t)(raw[2 * i] | (raw[2 * i + 1] << 8));
+    }
+    return axc_table_create(t.data(), out);
+}
+
+int axc_table_destroy(axc_table *table)
+{
+    if (!table)
+        return AXC_OK;
+    hipError_t e = hipFree(table->dev_tableT);
+    delete table;
+    if (e != hipSuccess)
+        return fail_hip(e, "hipFree");
+    return AXC_OK;
+}
+
+int axc_quant_props_compute(float input_min, float input_max, float filter_min, float filter_max,
+                            axc_quant_props *out)
+{
+    if (!out)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    var_quant_props(input_min, input_max, &out->input_scale, &out->input_inv_scale, &out->input_offset);
+    var_quant_props(filter_min, filter_max, &out->filter_scale, &out->filter_inv_scale, &out->filter_offset);
+    volatile float s = out->input_scale * out->filter_scale;
+    out->s1xs2 = s;
+    out->m1 = out->input_offset;
+    out->m2 = out->filter_offset;
+    volatile float mm = out->m1 * out->m2;
+    out->m1xm2 = mm;
+    out->input_zero_code = host_quantize(0.0f, out->input_offset, out->input_inv_scale);
+    return AXC_OK;
+}
+
+int axc_conv2d_geometry(const axc_conv2d_desc *desc, axc_conv2d_dims *dims) { return geometry(desc, dims); }
+
+int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes)
+{
+    if (!bytes)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    PreparedDense pd;
+    int rc = prepare_dense(desc, &pd);
+    if (rc != AXC_OK)
+        return rc;
+    *bytes = pd.ws.total;
+    return AXC_OK;
+}
+
+int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes)
+{
+    if (!bytes)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    axc_conv2d_dims dm;
+    int rc = geometry(desc, &dm);
+    if (rc != AXC_OK)
+        return rc;
+    rc = validate_for_launch(desc, dm, true);
+    if (rc != AXC_OK)
+        return rc;
+    *bytes = align_up((size_t)dm.filter_rows * dm.filter_cols * dm.in_depth) + align_up((size_t)dm.in_depth * 4);
+    return AXC_OK;
+}
+
+int axc_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                      const float *filter, float input_min, float input_max, float filter_min, float filter_max,
+                      float *output, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return run_dense(table, desc, input, filter, nullptr, nullptr, 0, input_min, input_max, filter_min,
+                     filter_max, output, nullptr, workspace, workspace_bytes, stream);
+}
+
+int axc_conv2d_minmax_acc_i32(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                              const float *filter, float input_min, float input_max, float filter_min,
+                              float filter_max, int32_t *acc, void *workspace, size_t workspace_bytes,
+                              void *stream)
+{
+    return run_dense(table, desc, input, filter, nullptr, nullptr, 0, input_min, input_max, filter_min,
+                     filter_max, nullptr, acc, workspace, workspace_bytes, stream);
+}
+
+int axc_conv2d_codes_acc_i32(const axc_table *table, const axc_conv2d_desc *desc, const uint8_t *input_codes,
+                             const uint8_t *filter_codes, int input_zero_code, int32_t *acc, void *workspace,
+                             size_t workspace_bytes, void *stream)
+{
+    if (!input_codes || !filter_codes) {
+        // distinguish "empty output" from a null pointer only after geometry
+        PreparedDense pd;
+        int rc = prepare_dense(desc, &pd);
+        if (rc != AXC_OK)
+            return rc;
+        if (pd.empty)
+            return AXC_OK;
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    }
+    return run_dense(table, desc, nullptr, nullptr, input_codes, filter_codes, input_zero_code, 0, 0, 0, 0,
+                     nullptr, acc, workspace, workspace_bytes, stream);
+}
+
+int axc_depthwise_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                                const float *filter, float input_min, float input_max, float filter_min,
+                                float filter_max, float *output, void *workspace, size_t workspace_bytes,
+                                void *stream)
+{
+    return run_depthwise(table, desc, input, filter, input_min, input_max, filter_min, filter_max, output,
+                         nullptr, workspace, workspace_bytes, stream);
+}
+
+int axc_depthwise_conv2d_minmax_acc_i32(const axc_table *table, const axc_conv2d_desc *desc,
+                                        const float *input, const float *filter, float input_min,
+                                        float input_max, float filter_min, float filter_max, int32_t *acc,
+                                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    return run_depthwise(table, desc, input, filter, input_min, input_max, filter_min, filter_max, nullptr, acc,
+                         workspace, workspace_bytes, stream);
+}
+
+int axc_quantize(const float *values, int64_t n, float min, float max, uint8_t *codes, void *stream)
+{
+    if (n < 0 || (n > 0 && (!values || !codes)))
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    float scale, inv, offset;
+    var_quant_props(min, max, &scale, &inv, &offset);
+    AXC_HIP(launch_quantize_flat(values, n, offset, inv, codes, static_cast<hipStream_t>(stream)));
+    return AXC_OK;
+}
+
+int axc_profile_enable(int enable)
+{
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    g_prof_enabled = enable != 0;
+    return AXC_OK;
+}
+
+int axc_profile_reset(void)
+{
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    for (auto &kv : g_prof)
+        prof_drain_locked(kv.second);
+    g_prof.clear();
+    return AXC_OK;
+}
+
+int axc_profile_read(int index, char *name, size_t name_bytes, double *total_ms, int64_t *launches)
+{
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (index < 0 || (size_t)index >= g_prof.size())
+        return AXC_INVALID_ARGUMENT; // end of list; not an error worth a message
+    auto it = g_prof.begin();
+    std::advance(it, index);
+    prof_drain_locked(it->second);
+    if (name && name_bytes) {
+        strncpy(name, it->first.c_str(), name_bytes - 1);
+        name[name_bytes - 1] = 0;
+    }
+    if (total_ms)
+        *total_ms = it->second.total_ms;
+    if (launches)
+        *launches = it->second.launches;
+    return AXC_OK;
+}
+
+int axc_lds_gather_peak(double *lookups_per_second, void *stream)
+{
+    if (!lookups_per_second)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    *lookups_per_second = 0.0;
+    AXC_HIP(run_lds_gather_peak(lookups_per_second, static_cast<hipStream_t>(stream)));
+    return AXC_OK;
+}
+
+int axc_device_info(int *compute_units, int *lds_bytes_per_workgroup, int *clock_khz)
+{
+    int dev = 0;
+    AXC_HIP(hipGetDevice(&dev));
+    int v = 0;
+    if (compute_units) {
+        AXC_HIP(hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev));
+        *compute_units = v;
+    }
+    if (lds_bytes_per_workgroup) {
+        AXC_HIP(hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+        *lds_bytes_per_workgroup = v;
+    }
+    if (clock_khz) {
+        AXC_HIP(hipDeviceGetAttribute(&v, hipDeviceAttributeClockRate, dev));
+        *clock_khz = v;
+    }
+    return AXC_OK;
+}
+
+} // extern "C"

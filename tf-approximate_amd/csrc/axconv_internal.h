@@ -1,0 +1,96 @@
+// Internal declarations shared by the HIP translation units of libaxconv_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "axconv.h"
+
+namespace axc {
+
+// LDS budget of one workgroup (the whole CU: 160 KiB).
+constexpr int kTableBytes = 131072;            // 256 x 256 uint16, weight-code major
+constexpr int kExpandBytes = 32768;            // 256 activation rows x 64 slots x uint16
+constexpr int kLdsBytes = kTableBytes + kExpandBytes;
+constexpr int kBlockThreads = 1024;            // 16 wavefronts: one workgroup per CU
+constexpr int kWaves = kBlockThreads / 64;
+constexpr uint16_t kNullWeight = 0xFFFF;       // slot that contributes nothing (padding channel / column)
+
+// Geometry of one dense layer after validation.
+struct ConvGeom {
+    int N, H, W, C;        // input NHWC
+    int KH, KW, Co;        // filter HWIO (in depth == C)
+    int OH, OW;
+    int sh, sw, dh, dw, ph, pw;
+    int C4;                // ceil(C / 4): channel quads in the quantized activation layout
+    int64_t M;             // N * OH * OW
+    int K;                 // KH * KW * C
+};
+
+// How the dense LUT-GEMM is cut into workgroup tiles.
+struct DensePlan {
+    int nt;                // columns per tile: 16, 32 or 64
+    int rows_per_tile;     // multiple of 64, <= 1024 * (64 / nt)
+    int n_row_tiles, n_col_tiles;
+    int fills;             // expanded-row refills per tile: KH*KW * C4 * (4 / (64/nt))
+    int grid;
+};
+
+struct DenseParams {
+    ConvGeom g;
+    DensePlan plan;
+    const uint32_t *xq;     // [N][H][C4][W] dwords of 4 row-permuted activation codes
+    const float *chsum;     // [N][H][W] sum over channels of the raw input (float epilogue only)
+    const uint16_t *wq;     // [n_col_tiles][fills][64] packed filter codes (kNullWeight = none)
+    const float *fsum;      // [Co] sum over (h, w, c) of the raw filter
+    const uint16_t *tableT; // [256 filter code][256 input code]
+    float *out_f;
+    int32_t *out_i;
+    float s1xs2, m1, m2, k_m1xm2; // epilogue constants; k_m1xm2 = float(K) * m1xM2
+    uint32_t zp4;           // row-permuted zero code replicated in all four bytes
+};
+
+struct DepthwiseParams {
+    int N, H, W, C, KH, KW, OH, OW, sh, sw, dh, dw, ph, pw;
+    int64_t M;
+    const float *x;         // NHWC raw input
+    const uint8_t *wcodes;  // [KH*KW][C] filter codes
+    const float *fsum;      // [C]
+    const uint16_t *tableT;
+    float *out_f;
+    int32_t *out_i;
+    float in_offset, in_inv_scale;
+    float s1xs2, m1, m2, k_m1xm2;
+};
+
+// Row permutation of the expanded table: logical activation code a lives in physical row
+// (a >> 2) | ((a & 3) << 6), so that the four codes one lane transposes land in rows of
+// alternating bank parity.
+__host__ __device__ inline uint32_t phys_row(uint32_t a) { return (a >> 2) | ((a & 3u) << 6); }
+
+// Device-side quantize: three separately rounded fp32 operations, truncation, clamp.
+__device__ inline uint32_t quantize_code(float v, float offset, float inv_scale)
+{
+    float t = __fadd_rn(__fmul_rn(__fsub_rn(v, offset), inv_scale), 0.5f);
+    t = t > 0.0f ? t : 0.0f;          // also maps NaN to 0
+    t = t < 255.0f ? t : 255.0f;      // truncation of [255,256) is 255 as well
+    return (uint32_t)t;
+}
+
+// ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
+hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
+                                    uint32_t *xq, float *chsum, hipStream_t stream);
+hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t *xq, hipStream_t stream);
+hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
+                              const DensePlan &plan, float offset, float inv_scale,
+                              uint16_t *wq, float *fsum, hipStream_t stream);
+hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
+                                hipStream_t stream);
+hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream);
+hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
+                                   uint8_t *wcodes, float *fsum, hipStream_t stream);
+hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream);
+hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream);
+
+} // namespace axc

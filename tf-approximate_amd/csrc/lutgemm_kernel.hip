@@ -1,0 +1,293 @@
+// Dense LUT-GEMM for gfx950: implicit-GEMM gather + table lookups out of LDS + fused epilogue.
+//
+// One workgroup (16 wavefronts) owns a CU and its 160 KiB of LDS:
+//   [0, 128 KiB)        the whole truth table, weight-code major: row b holds T[a][b] for a = 0..255
+//   [128 KiB, 160 KiB)  the "expanded rows": for the 64 weight slots of the current fill,
+//                       E[phys_row(a)][slot] = T[a][code(slot)], 128 bytes per activation code
+//
+// A fill takes 64 filter entries (KS consecutive input channels x NT output columns, KS * NT = 64),
+// copies the table row of each entry into the expanded area transposed (derive phase), then every
+// lane looks up, for each of its R = 64 / NT output pixels, the expanded row of its activation code
+// with ds_read_b128: eight table entries per LDS access instead of one, and the 16-byte chunks the
+// lanes of a wavefront touch in one instruction are rotated by lane so they fall into different
+// banks whatever the activation codes are.  Sums are exact int32.
+//
+// Restates, as one fused kernel, what the reference does in ApproxConvIm2ColKernel +
+// ApproxConvGEMMKernel (tf2/src/approx_nn_conv_kernels.cpp:215-296) per chunk.
+#include "axconv_internal.h"
+
+namespace axc {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+extern __shared__ __align__(16) unsigned char lds[];
+
+template <int NT, bool OUT_I32>
+__global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const DenseParams p)
+{
+    constexpr int R = 64 / NT;        // output pixels per lane
+    constexpr int KS = 64 / NT;       // input channels per fill
+    constexpr int SETS = NT / 8;      // 8-column groups per pixel
+    constexpr int SUBS = 4 / KS;      // fills per channel quad
+    constexpr int LOG_SETS = (SETS == 8) ? 3 : (SETS == 4) ? 2 : 1;
+
+    const ConvGeom &g = p.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+
+    // ---- stage the truth table (once per workgroup; the workgroup is persistent) ----
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(p.tableT);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
+#pragma unroll
+        for (int i = 0; i < kTableBytes / 16 / kBlockThreads; ++i)
+            dst[tid + i * kBlockThreads] = src[tid + i * kBlockThreads];
+    }
+
+    // ---- lane constants ----
+    const int c0 = lane & 7;
+    uint32_t choff[8];   // byte offset of the chunk this lane reads at step s
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        choff[s] = (uint32_t)kTableBytes + ((uint32_t)((c0 + s) & 7) << 4);
+    // The chunk of step s belongs to input channel kk_s = ((c0 + s) & 7) >> LOG_SETS of the fill.
+    // KS == 4: kk_s = (kk0 + ((p0 + s) >> 1)) & 3 with kk0 = c0 >> 1, p0 = c0 & 1, so after rotating the
+    //          activation dword right by kk0 bytes (and by p0 more for odd s) the byte index is the
+    //          compile-time constant s >> 1.
+    // KS == 2: kk_s is one bit; it is kept as a per-step lane mask.
+    const uint32_t rot_kk0 = (uint32_t)(c0 >> 1) << 3;
+    const uint32_t rot_p0 = (uint32_t)(c0 & 1) << 3;
+    bool kk_hi[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        kk_hi[s] = ((((c0 + s) & 7) >> LOG_SETS) & 1) != 0;
+    // derive phase: lane transposes activation codes 4*lane .. 4*lane+3 for slots 4*jq .. 4*jq+3
+    const int jq = (lane + wave) & 15;
+    const uint32_t rd_off = (uint32_t)lane * 8u;
+    const uint32_t wr_off = (uint32_t)kTableBytes + (uint32_t)lane * 128u + (uint32_t)jq * 8u;
+
+    const int taps = g.KH * g.KW;
+    const int ntiles = p.plan.n_row_tiles * p.plan.n_col_tiles;
+    const int fills = p.plan.fills;
+
+    for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int ct = tile % p.plan.n_col_tiles;
+        const int rt = tile / p.plan.n_col_tiles;
+        const int64_t row0 = (int64_t)rt * p.plan.rows_per_tile;
+        const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
+
+        // ---- per-pixel geometry ----
+        int32_t nbase[R];  // dword index of (n, 0, 0, 0) in xq
+        int hw0[R];        // (ih0 << 16) | (iw0 & 0xffff): input coordinates of tap (0, 0)
+        bool rvalid[R];    // this lane's pixel exists
+        bool ractive[R];   // some lane of this wavefront has a pixel (wave-uniform)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t wrow = row0 + (int64_t)(r * kWaves + wave) * 64;
+            ractive[r] = wrow < row_end;
+            const int64_t m = wrow + lane;
+            rvalid[r] = m < row_end;
+            const int64_t mm = rvalid[r] ? m : row0;
+            const int n = (int)(mm / ((int64_t)g.OH * g.OW));
+            const int rem = (int)(mm - (int64_t)n * g.OH * g.OW);
+            const int oh = rem / g.OW;
+            const int ow = rem - oh * g.OW;
+            nbase[r] = n * g.H * g.C4 * g.W;
+            hw0[r] = ((oh * g.sh - g.ph) << 16) | ((ow * g.sw - g.pw) & 0xffff);
+        }
+
+        int32_t acc[R][NT];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+                acc[r][j] = 0;
+
+        const uint16_t *wq_tile = p.wq + (size_t)ct * fills * 64;
+
+        // ---- software pipeline: the loads of the next channel quad / next fill are issued
+        //      before the current fill's LDS work ----
+        int32_t base_n[R]; // dword index of the next quad to load, valid if inb_n
+        bool inb_n[R];
+        int tap_n = 0, q_n = 0, kh_n = 0, kw_n = 0;
+        auto tap_setup = [&]() {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int ih = (hw0[r] >> 16) + kh_n * g.dh;
+                const int iw = (int)(int16_t)(hw0[r] & 0xffff) + kw_n * g.dw;
+                inb_n[r] = rvalid[r] && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+                base_n[r] = nbase[r] + ih * g.C4 * g.W + iw;
+            }
+        };
+        uint32_t a4n[R];
+        auto issue_act_loads = [&]() {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                a4n[r] = inb_n[r] ? p.xq[base_n[r] + q_n * g.W] : p.zp4;
+        };
+        tap_setup();
+        issue_act_loads();
+        u32x2 wn = *reinterpret_cast<const u32x2 *>(wq_tile + jq * 4);
+
+        int fill = 0;
+        for (int tap = 0; tap < taps; ++tap) {
+            for (int q = 0; q < g.C4; ++q) {
+                uint32_t a4[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    a4[r] = a4n[r];
+                // advance the load cursor and issue the next quad's loads
+                if (++q_n == g.C4) {
+                    q_n = 0;
+                    ++tap_n;
+                    if (++kw_n == g.KW) { kw_n = 0; ++kh_n; }
+                    if (tap_n < taps)
+                        tap_setup();
+                }
+                if (tap_n < taps)
+                    issue_act_loads();
+
+#pragma unroll
+                for (int sub = 0; sub < SUBS; ++sub, ++fill) {
+                    const u32x2 wc = wn;
+                    if (fill + 1 < fills)
+                        wn = *reinterpret_cast<const u32x2 *>(wq_tile + (size_t)(fill + 1) * 64 + jq * 4);
+
+                    // ---- derive: expanded rows for this fill's 64 slots ----
+                    __syncthreads(); // previous fill's lookups (and the table staging) are done
+                    {
+                        uint32_t code[4] = {wc.x & 0xffffu, wc.x >> 16, wc.y & 0xffffu, wc.y >> 16};
+                        u32x2 v[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const bool none = code[i] == kNullWeight;
+                            const uint32_t row = none ? 0u : code[i];
+                            v[i] = *reinterpret_cast<const u32x2 *>(lds + row * 512u + rd_off);
+                            if (none) { v[i].x = 0u; v[i].y = 0u; }
+                        }
+                        u32x2 o[4];
+                        o[0].x = __builtin_amdgcn_perm(v[1].x, v[0].x, 0x05040100u);
+                        o[0].y = __builtin_amdgcn_perm(v[3].x, v[2].x, 0x05040100u);
+                        o[1].x = __builtin_amdgcn_perm(v[1].x, v[0].x, 0x07060302u);
+                        o[1].y = __builtin_amdgcn_perm(v[3].x, v[2].x, 0x07060302u);
+                        o[2].x = __builtin_amdgcn_perm(v[1].y, v[0].y, 0x05040100u);
+                        o[2].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x05040100u);
+                        o[3].x = __builtin_amdgcn_perm(v[1].y, v[0].y, 0x07060302u);
+                        o[3].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x07060302u);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            *reinterpret_cast<u32x2 *>(lds + wr_off + (uint32_t)i * (64u * 128u)) = o[i];
+                    }
+                    __syncthreads();
+
+                    // ---- lookups ----
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        if (!ractive[r])
+                            continue;
+                        // row offsets (128 B per activation code) of the channels of this fill
+                        uint32_t ax = 0, ay = 0;
+                        if (KS == 1) {
+                            ax = ((a4[r] >> (8 * sub)) & 0xffu) << 7;
+                        } else if (KS == 2) {
+                            ax = ((a4[r] >> (16 * sub)) & 0xffu) << 7;
+                            ay = ((a4[r] >> (16 * sub + 8)) & 0xffu) << 7;
+                        } else {
+                            ax = __builtin_amdgcn_alignbit(a4[r], a4[r], rot_kk0);
+                            ay = __builtin_amdgcn_alignbit(ax, ax, rot_p0);
+                        }
+#pragma unroll
+                        for (int s = 0; s < 8; ++s) {
+                            uint32_t aoff;
+                            if (KS == 1)
+                                aoff = ax;
+                            else if (KS == 2)
+                                aoff = kk_hi[s] ? ay : ax;
+                            else
+                                aoff = ((((s & 1) ? ay : ax) >> (8 * (s >> 1))) & 0xffu) << 7;
+                            const u32x4 e = *reinterpret_cast<const u32x4 *>(lds + aoff + choff[s]);
+                            int32_t *a = &acc[r][(s & (SETS - 1)) * 8];
+                            a[0] += (int32_t)(e.x & 0xffffu);
+                            a[1] += (int32_t)(e.x >> 16);
+                            a[2] += (int32_t)(e.y & 0xffffu);
+                            a[3] += (int32_t)(e.y >> 16);
+                            a[4] += (int32_t)(e.z & 0xffffu);
+                            a[5] += (int32_t)(e.z >> 16);
+                            a[6] += (int32_t)(e.w & 0xffffu);
+                            a[7] += (int32_t)(e.w >> 16);
+                        }
+                    }
+                }
+            }
+        }
+
+        // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!rvalid[r])
+                continue;
+            const int64_t m = row0 + (int64_t)(r * kWaves + wave) * 64 + lane;
+            float psum = 0.0f;
+            if (!OUT_I32) {
+                // patch sum = sum over taps of the per-pixel channel sums (0 outside the image)
+                const int n = (int)(m / ((int64_t)g.OH * g.OW));
+                const int ih0 = hw0[r] >> 16;
+                const int iw0 = (int)(int16_t)(hw0[r] & 0xffff);
+                for (int kh = 0; kh < g.KH; ++kh)
+                    for (int kw = 0; kw < g.KW; ++kw) {
+                        const int ih = ih0 + kh * g.dh, iw = iw0 + kw * g.dw;
+                        if ((unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
+                            psum = __fadd_rn(psum, p.chsum[((int64_t)n * g.H + ih) * g.W + iw]);
+                    }
+            }
+            const float t1 = __fmul_rn(p.m2, psum);
+#pragma unroll
+            for (int set = 0; set < SETS; ++set) {
+                const int h = (c0 + set) & (SETS - 1);
+                const int col0 = ct * NT + h * 8;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int col = col0 + e;
+                    if (col >= g.Co)
+                        continue;
+                    const int32_t a = acc[r][set * 8 + e];
+                    if (OUT_I32) {
+                        p.out_i[m * g.Co + col] = a;
+                    } else {
+                        const float t0 = __fmul_rn((float)a, p.s1xs2);
+                        const float t2 = __fadd_rn(t0, t1);
+                        const float t3 = __fmul_rn(p.m1, p.fsum[col]);
+                        const float t4 = __fadd_rn(t2, t3);
+                        p.out_f[m * g.Co + col] = __fsub_rn(t4, p.k_m1xm2);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int NT, bool OUT_I32>
+static hipError_t launch_one(const DenseParams &p, hipStream_t stream)
+{
+    auto kernel = lutgemm_expand_kernel<NT, OUT_I32>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kernel, dim3(p.plan.grid), dim3(kBlockThreads), kLdsBytes, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream)
+{
+    switch (p.plan.nt) {
+    case 16: return out_i32 ? launch_one<16, true>(p, stream) : launch_one<16, false>(p, stream);
+    case 32: return out_i32 ? launch_one<32, true>(p, stream) : launch_one<32, false>(p, stream);
+    case 64: return out_i32 ? launch_one<64, true>(p, stream) : launch_one<64, false>(p, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+} // namespace axc

@@ -1,0 +1,193 @@
+// Pre-pass kernels: quantize + relayout of the input, filter quantize/pack/sums, flat quantize.
+#include "axconv_internal.h"
+
+namespace axc {
+
+// Input pre-pass.  Restates the quantize and the channel part of the patch sum of
+// ApproxConvIm2ColKernel (tf2/src/approx_nn_conv_kernels.cpp:288-294) once per input element
+// instead of once per patch element.
+//   xq   [N][H][C4][W]  one dword = codes of channels 4*c4 .. 4*c4+3 of one pixel, each code stored as
+//                       its expanded-row index phys_row(code)
+//   chsum[N][H][W]      sum over channels of the raw floats, c ascending
+// One thread per pixel: the channel loop is sequential so the sum has the reference's order within a pixel.
+__global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__restrict__ x, int64_t pixels,
+                                                                 int H, int W, int C, int C4, float offset,
+                                                                 float inv_scale, uint32_t *__restrict__ xq,
+                                                                 float *__restrict__ chsum)
+{
+    const int64_t pix = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (pix >= pixels)
+        return;
+    const int w = (int)(pix % W);
+    const int64_t nh = pix / W; // n * H + h
+    const float *src = x + pix * C;
+    float sum = 0.0f;
+    for (int c4 = 0; c4 < C4; ++c4) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = c4 * 4 + i;
+            if (c < C) {
+                const float v = src[c];
+                sum = __fadd_rn(sum, v);
+                packed |= phys_row(quantize_code(v, offset, inv_scale)) << (8 * i);
+            }
+        }
+        xq[(nh * C4 + c4) * W + w] = packed;
+    }
+    if (chsum)
+        chsum[pix] = sum;
+}
+
+// Same relayout for caller-supplied codes (uint8 NHWC).
+__global__ void __launch_bounds__(256) codes_relayout_kernel(const uint8_t *__restrict__ codes, int64_t pixels,
+                                                              int W, int C, int C4, uint32_t *__restrict__ xq)
+{
+    const int64_t pix = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (pix >= pixels)
+        return;
+    const int w = (int)(pix % W);
+    const int64_t nh = pix / W;
+    const uint8_t *src = codes + pix * C;
+    for (int c4 = 0; c4 < C4; ++c4) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = c4 * 4 + i;
+            if (c < C)
+                packed |= phys_row(src[c]) << (8 * i);
+        }
+        xq[(nh * C4 + c4) * W + w] = packed;
+    }
+}
+
+// Filter pre-pass: quantize (tf2/src/approx_nn_conv_kernels.cpp:243, hoisted out of the GEMM loop)
+// and pack into the order the LUT-GEMM consumes.
+//   wq[ct][fill][slot], fill = (tap * C4 + q) * SUBS + sub, slot = kk * NT + j
+//   channel = q*4 + sub*KS + kk, column = ct*NT + j; kNullWeight where channel >= C or column >= Co.
+__global__ void __launch_bounds__(256) filter_pack_kernel(const float *__restrict__ filter,
+                                                           const uint8_t *__restrict__ filter_codes, int taps,
+                                                           int C, int C4, int Co, int nt, int n_col_tiles,
+                                                           float offset, float inv_scale,
+                                                           uint16_t *__restrict__ wq)
+{
+    const int ks = 64 / nt, subs = 4 / ks;
+    const int fills = taps * C4 * subs;
+    const int64_t total = (int64_t)n_col_tiles * fills * 64;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total)
+        return;
+    const int slot = (int)(i & 63);
+    const int64_t f = i >> 6;
+    const int fill = (int)(f % fills);
+    const int ct = (int)(f / fills);
+    const int sub = fill % subs;
+    const int tq = fill / subs;
+    const int q = tq % C4;
+    const int tap = tq / C4;
+    const int kk = slot / nt, j = slot % nt;
+    const int c = q * 4 + sub * ks + kk;
+    const int col = ct * nt + j;
+    uint16_t code = kNullWeight;
+    if (c < C && col < Co) {
+        const int64_t idx = ((int64_t)tap * C + c) * Co + col;
+        code = filter_codes ? (uint16_t)filter_codes[idx]
+                            : (uint16_t)quantize_code(filter[idx], offset, inv_scale);
+    }
+    wq[i] = code;
+}
+
+// Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one thread per output column,
+// rows (h, w, c) ascending.
+__global__ void __launch_bounds__(256) filter_sums_kernel(const float *__restrict__ filter, int K, int Co,
+                                                           float *__restrict__ fsum)
+{
+    const int col = blockIdx.x * blockDim.x + threadIdx.x;
+    if (col >= Co)
+        return;
+    float s = 0.0f;
+    for (int k = 0; k < K; ++k)
+        s = __fadd_rn(s, filter[(int64_t)k * Co + col]);
+    fsum[col] = s;
+}
+
+__global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
+                                                             float inv_scale, uint8_t *__restrict__ codes)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        codes[i] = (uint8_t)quantize_code(v[i], offset, inv_scale);
+}
+
+// Depthwise filter pre-pass: codes [taps][C] and per-channel sums (taps ascending).
+__global__ void __launch_bounds__(256) depthwise_filter_kernel(const float *__restrict__ filter, int taps, int C,
+                                                                float offset, float inv_scale,
+                                                                uint8_t *__restrict__ wcodes,
+                                                                float *__restrict__ fsum)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C)
+        return;
+    float s = 0.0f;
+    for (int t = 0; t < taps; ++t) {
+        const float v = filter[(int64_t)t * C + c];
+        s = __fadd_rn(s, v);
+        wcodes[(int64_t)t * C + c] = (uint8_t)quantize_code(v, offset, inv_scale);
+    }
+    fsum[c] = s;
+}
+
+static inline unsigned blocks_for(int64_t n, int threads) { return (unsigned)((n + threads - 1) / threads); }
+
+hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
+                                    uint32_t *xq, float *chsum, hipStream_t stream)
+{
+    const int64_t pixels = (int64_t)g.N * g.H * g.W;
+    hipLaunchKernelGGL(quantize_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, x, pixels,
+                       g.H, g.W, g.C, g.C4, offset, inv_scale, xq, chsum);
+    return hipGetLastError();
+}
+
+hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t *xq, hipStream_t stream)
+{
+    const int64_t pixels = (int64_t)g.N * g.H * g.W;
+    hipLaunchKernelGGL(codes_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, codes, pixels,
+                       g.W, g.C, g.C4, xq);
+    return hipGetLastError();
+}
+
+hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
+                              const DensePlan &plan, float offset, float inv_scale, uint16_t *wq, float *fsum,
+                              hipStream_t stream)
+{
+    const int64_t total = (int64_t)plan.n_col_tiles * plan.fills * 64;
+    hipLaunchKernelGGL(filter_pack_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, stream, filter,
+                       filter_codes, g.KH * g.KW, g.C, g.C4, g.Co, plan.nt, plan.n_col_tiles, offset, inv_scale,
+                       wq);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !fsum || !filter)
+        return e;
+    hipLaunchKernelGGL(filter_sums_kernel, dim3(blocks_for(g.Co, 256)), dim3(256), 0, stream, filter, g.K, g.Co,
+                       fsum);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
+                                hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    hipLaunchKernelGGL(quantize_flat_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream, v, n, offset,
+                       inv_scale, codes);
+    return hipGetLastError();
+}
+
+hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
+                                   uint8_t *wcodes, float *fsum, hipStream_t stream)
+{
+    hipLaunchKernelGGL(depthwise_filter_kernel, dim3(blocks_for(C, 256)), dim3(256), 0, stream, filter, taps, C,
+                       offset, inv_scale, wcodes, fsum);
+    return hipGetLastError();
+}
+
+} // namespace axc

@@ -1,0 +1,296 @@
+"""Python face of the op, mirroring the wrapper TensorFlow generates for the reference's
+REGISTER_OP("ApproxConv2DWithMinMaxVars") (tf2/src/approx_nn_ops.cpp:38-54): same argument names,
+order and meaning as the call in tf2/test/test_table_approx_conv_2d.py:47-49.
+
+Tensors are torch tensors on a ROCm device (torch is only the owner of device memory and of the
+stream); all arithmetic happens in libaxconv_hip.so.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+
+class InvalidArgumentError(ValueError):
+    """tensorflow::errors::InvalidArgument in the reference."""
+
+
+class UnimplementedError(NotImplementedError):
+    """tensorflow::errors::Unimplemented in the reference."""
+
+
+def _check(rc):
+    if rc == _lib.OK:
+        return
+    msg = _lib.load().axc_last_error().decode()
+    if rc == _lib.INVALID_ARGUMENT:
+        raise InvalidArgumentError(msg)
+    if rc == _lib.UNIMPLEMENTED:
+        raise UnimplementedError(msg)
+    raise RuntimeError(msg)
+
+
+_PADDING = {"VALID": _lib.PAD_VALID, "SAME": _lib.PAD_SAME, "EXPLICIT": _lib.PAD_EXPLICIT}
+_FORMAT = {"NHWC": _lib.FORMAT_NHWC, "NCHW": _lib.FORMAT_NCHW}
+
+
+def make_desc(input_shape, filter_shape, strides, padding, explicit_paddings=(), data_format="NHWC",
+              dilations=(1, 1, 1, 1), num_bits=8):
+    if len(input_shape) != 4:
+        raise InvalidArgumentError("input must be 4-dimensional")
+    if len(filter_shape) != 4:
+        raise InvalidArgumentError("filter must be 4-dimensional")
+    if len(strides) != 4:
+        raise InvalidArgumentError("Sliding window strides must specify 4 dimensions")
+    if len(dilations) != 4:
+        raise InvalidArgumentError("Sliding window dilations field must specify 4 dimensions")
+    if isinstance(padding, bytes):
+        padding = padding.decode()
+    if padding not in _PADDING:
+        raise InvalidArgumentError("Invalid padding")
+    if data_format not in _FORMAT:
+        raise InvalidArgumentError("Invalid data format")
+    d = _lib.ConvDesc()
+    for i in range(4):
+        d.input_shape[i] = int(input_shape[i])
+        d.filter_shape[i] = int(filter_shape[i])
+        d.strides[i] = int(strides[i])
+        d.dilations[i] = int(dilations[i])
+    d.padding = _PADDING[padding]
+    d.data_format = _FORMAT[data_format]
+    d.num_bits = int(num_bits)
+    ep = list(explicit_paddings) + [0] * 8
+    for i in range(8):
+        d.explicit_paddings[i] = int(ep[i])
+    return d
+
+
+def conv2d_geometry(desc):
+    dims = _lib.ConvDims()
+    _check(_lib.load().axc_conv2d_geometry(ctypes.byref(desc), ctypes.byref(dims)))
+    return dims
+
+
+def quant_props(input_min, input_max, filter_min, filter_max):
+    qp = _lib.QuantProps()
+    _check(_lib.load().axc_quant_props_compute(float(input_min), float(input_max), float(filter_min),
+                                               float(filter_max), ctypes.byref(qp)))
+    return qp
+
+
+class TruthTable:
+    """Device-resident 256x256 uint16 truth table (the op's `mul_map_file` attr, loaded once)."""
+
+    def __init__(self, source="", num_bits=8):
+        lib = _lib.load()
+        handle = ctypes.c_void_p()
+        if isinstance(source, (str, bytes)):
+            name = source.encode() if isinstance(source, str) else source
+            _check(lib.axc_table_create_from_file(name, int(num_bits), ctypes.byref(handle)))
+        else:
+            import numpy as np
+            if int(num_bits) != 8:
+                raise InvalidArgumentError("only num_bits = 8 is supported")
+            host = np.ascontiguousarray(source, dtype=np.uint16).reshape(-1)
+            if host.size != 65536:
+                raise InvalidArgumentError("truth table must hold 65536 uint16 entries")
+            _check(lib.axc_table_create(host.ctypes.data, ctypes.byref(handle)))
+        self.handle = handle
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                _lib.load().axc_table_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    buf = _workspaces.get(device)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _workspaces[device] = buf
+    return buf
+
+
+def _scalar(v):
+    if torch.is_tensor(v):
+        return float(v.item())
+    return float(v)
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_device_f32(t, what):
+    if not torch.is_tensor(t) or not t.is_cuda:
+        raise InvalidArgumentError("%s must be a tensor on the GPU" % what)
+    if t.dtype != torch.float32:
+        raise UnimplementedError("%s: only float32 is registered for this op" % what)
+    return t.contiguous()
+
+
+class ApproxConv2DWithMinMaxVars:
+    """One op instance: attrs fixed at construction, like the reference's OpKernel
+    (ApproxConv2DOp, tf2/src/approx_nn_conv_ops.cpp:411-468)."""
+
+    def __init__(self, strides, num_bits, mul_map_file, padding, explicit_paddings=(), data_format="NHWC",
+                 dilations=(1, 1, 1, 1), depthwise=False):
+        self.strides = list(strides)
+        self.num_bits = int(num_bits)
+        self.padding = padding
+        self.explicit_paddings = list(explicit_paddings)
+        self.data_format = data_format
+        self.dilations = list(dilations)
+        self.depthwise = depthwise
+        self.table = mul_map_file if isinstance(mul_map_file, TruthTable) else TruthTable(mul_map_file, num_bits)
+        # attr checks the reference performs at construction (InitApproxConv2DParameters)
+        make_desc((1, 1, 1, 1), (1, 1, 1, 1), self.strides, self.padding, self.explicit_paddings,
+                  self.data_format, self.dilations, self.num_bits)
+
+    def _desc(self, input, filter):
+        return make_desc(tuple(input.shape), tuple(filter.shape), self.strides, self.padding,
+                         self.explicit_paddings, self.data_format, self.dilations, self.num_bits)
+
+    def _out_shape(self, dims):
+        depth = dims.in_depth if self.depthwise else dims.out_depth
+        return (dims.batch, int(dims.out_rows), int(dims.out_cols), depth)
+
+    def _run(self, input, filter, mins, acc_i32):
+        lib = _lib.load()
+        input = _require_device_f32(input, "input")
+        filter = _require_device_f32(filter, "filter")
+        desc = self._desc(input, filter)
+        dims = conv2d_geometry(desc)
+        nbytes = ctypes.c_size_t()
+        ws_fn = lib.axc_depthwise_conv2d_workspace_bytes if self.depthwise else lib.axc_conv2d_workspace_bytes
+        _check(ws_fn(ctypes.byref(desc), ctypes.byref(nbytes)))
+        ws = _workspace(input.device, nbytes.value)
+        out = torch.empty(self._out_shape(dims), dtype=torch.int32 if acc_i32 else torch.float32,
+                          device=input.device)
+        if self.depthwise:
+            fn = lib.axc_depthwise_conv2d_minmax_acc_i32 if acc_i32 else lib.axc_depthwise_conv2d_minmax
+        else:
+            fn = lib.axc_conv2d_minmax_acc_i32 if acc_i32 else lib.axc_conv2d_minmax
+        with torch.cuda.device(input.device):
+            _check(fn(self.table.handle, ctypes.byref(desc), input.data_ptr(), filter.data_ptr(),
+                      *[_scalar(m) for m in mins], out.data_ptr(), ws.data_ptr(), ws.numel(),
+                      _stream_ptr(input.device)))
+        return out
+
+    def __call__(self, input, filter, input_min, input_max, filter_min, filter_max):
+        return self._run(input, filter, (input_min, input_max, filter_min, filter_max), False)
+
+    def accumulators(self, input, filter, input_min, input_max, filter_min, filter_max):
+        """int32 sums of table entries before the epilogue (parity entry point)."""
+        return self._run(input, filter, (input_min, input_max, filter_min, filter_max), True)
+
+
+_table_cache = {}
+
+
+def _cached_table(mul_map_file, num_bits):
+    if isinstance(mul_map_file, TruthTable):
+        return mul_map_file
+    if not isinstance(mul_map_file, (str, bytes)):
+        return TruthTable(mul_map_file, num_bits)
+    key = (mul_map_file, int(num_bits))
+    if key not in _table_cache:
+        _table_cache[key] = TruthTable(mul_map_file, num_bits)
+    return _table_cache[key]
+
+
+def approx_conv2d_with_min_max_vars(input, filter, input_min, input_max, filter_min, filter_max, strides,
+                                    num_bits, mul_map_file, padding, explicit_paddings=(), data_format="NHWC",
+                                    dilations=(1, 1, 1, 1), name=None):
+    """Drop-in for the generated wrapper of the reference op (argument order of
+    tf2/test/test_table_approx_conv_2d.py:47-49).  mul_map_file may also be a TruthTable or a
+    uint16[65536] array, so seeded synthetic tables need no file."""
+    op = ApproxConv2DWithMinMaxVars(strides, num_bits, _cached_table(mul_map_file, num_bits), padding,
+                                    explicit_paddings, data_format, dilations)
+    return op(input, filter, input_min, input_max, filter_min, filter_max)
+
+
+def approx_depthwise_conv2d_with_min_max_vars(input, filter, input_min, input_max, filter_min, filter_max,
+                                              strides, num_bits, mul_map_file, padding, explicit_paddings=(),
+                                              data_format="NHWC", dilations=(1, 1, 1, 1), name=None):
+    """Depthwise variant (filter [rows, cols, C, 1]); the reference has no such op."""
+    op = ApproxConv2DWithMinMaxVars(strides, num_bits, _cached_table(mul_map_file, num_bits), padding,
+                                    explicit_paddings, data_format, dilations, depthwise=True)
+    return op(input, filter, input_min, input_max, filter_min, filter_max)
+
+
+def quantize(values, vmin, vmax):
+    """uint8 codes of a float32 device tensor (parity entry point for the quantize expression)."""
+    values = _require_device_f32(values, "values")
+    codes = torch.empty(values.shape, dtype=torch.uint8, device=values.device)
+    with torch.cuda.device(values.device):
+        _check(_lib.load().axc_quantize(values.data_ptr(), values.numel(), float(vmin), float(vmax),
+                                        codes.data_ptr(), _stream_ptr(values.device)))
+    return codes
+
+
+def conv2d_codes_acc_i32(table, input_codes, filter_codes, input_zero_code, strides=(1, 1, 1, 1),
+                         padding="SAME", dilations=(1, 1, 1, 1)):
+    """int32 LUT-GEMM sums on caller-supplied uint8 codes (NHWC / HWIO device tensors)."""
+    lib = _lib.load()
+    if input_codes.dtype != torch.uint8 or filter_codes.dtype != torch.uint8:
+        raise InvalidArgumentError("codes must be uint8")
+    input_codes = input_codes.contiguous()
+    filter_codes = filter_codes.contiguous()
+    desc = make_desc(tuple(input_codes.shape), tuple(filter_codes.shape), strides, padding, (), "NHWC", dilations)
+    dims = conv2d_geometry(desc)
+    nbytes = ctypes.c_size_t()
+    _check(lib.axc_conv2d_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+    ws = _workspace(input_codes.device, nbytes.value)
+    out = torch.empty((dims.batch, int(dims.out_rows), int(dims.out_cols), dims.out_depth), dtype=torch.int32,
+                      device=input_codes.device)
+    with torch.cuda.device(input_codes.device):
+        _check(lib.axc_conv2d_codes_acc_i32(table.handle, ctypes.byref(desc), input_codes.data_ptr(),
+                                            filter_codes.data_ptr(), int(input_zero_code), out.data_ptr(),
+                                            ws.data_ptr(), ws.numel(), _stream_ptr(input_codes.device)))
+    return out
+
+
+# ---- measurement helpers ---------------------------------------------------------------------
+
+def profile_enable(on=True):
+    _check(_lib.load().axc_profile_enable(1 if on else 0))
+
+
+def profile_reset():
+    _check(_lib.load().axc_profile_reset())
+
+
+def profile_read():
+    """{kernel name: (total_ms, launches)} since the last reset."""
+    lib = _lib.load()
+    out = {}
+    i = 0
+    while True:
+        name = ctypes.create_string_buffer(64)
+        ms = ctypes.c_double()
+        n = ctypes.c_int64()
+        if lib.axc_profile_read(i, name, 64, ctypes.byref(ms), ctypes.byref(n)) != _lib.OK:
+            break
+        out[name.value.decode()] = (ms.value, n.value)
+        i += 1
+    return out
+
+
+def lds_gather_peak():
+    v = ctypes.c_double()
+    _check(_lib.load().axc_lds_gather_peak(ctypes.byref(v), None))
+    return v.value
+
+
+def device_info():
+    a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _check(_lib.load().axc_device_info(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    return {"compute_units": a.value, "lds_bytes_per_workgroup": b.value, "clock_khz": c.value}
