@@ -1,0 +1,281 @@
+"""GPU parity: the HIP path (called through the C ABI) against the CPU oracle on identical inputs.
+Bars: int32 accumulators bit-exact; float outputs within 1e-5 max-normalized Linf (the reference test's
+own norm, tf2/test/test_table_approx_conv_2d.py:62)."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_util
+import refimpl
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+MM = (-1.0, 1.0, -0.5, 0.5)
+
+SMALL = [
+    # x_shape, f_shape, strides, padding, dilations, minmax
+    ((1, 8, 8, 4), (3, 3, 4, 6), (1, 1), "SAME", (1, 1), MM),
+    ((2, 9, 7, 3), (3, 3, 3, 5), (1, 1), "VALID", (1, 1), MM),
+    ((2, 11, 10, 5), (3, 2, 5, 7), (2, 2), "SAME", (1, 1), MM),
+    ((1, 12, 13, 2), (3, 3, 2, 4), (1, 2), "SAME", (2, 2), MM),
+    ((1, 12, 13, 2), (3, 3, 2, 4), (1, 1), "VALID", (2, 1), MM),
+    ((3, 6, 6, 8), (1, 1, 8, 9), (1, 1), "SAME", (1, 1), MM),          # reference's 1x1 path
+    ((2, 6, 6, 8), (1, 1, 8, 9), (2, 2), "VALID", (1, 1), MM),
+    ((4, 5, 4, 3), (5, 4, 3, 6), (1, 1), "VALID", (1, 1), MM),          # reference's filter == image path
+    ((1, 10, 10, 1), (8, 8, 1, 1), (1, 1), "SAME", (1, 1), (0.0, 1.0, 0.0, 1.0)),
+    ((1, 9, 9, 1), (3, 3, 1, 1), (1, 1), "SAME", (1, 1), (0.0, 6.0, -0.2, 0.1)),
+    ((2, 7, 7, 17), (3, 3, 17, 33), (1, 1), "SAME", (1, 1), MM),        # ragged channels / columns
+    ((1, 5, 5, 130), (3, 3, 130, 70), (2, 1), "SAME", (1, 1), MM),
+    ((1, 3, 3, 512), (3, 3, 512, 20), (1, 1), "SAME", (1, 1), MM),      # K = 4608: sums above 2^24
+    ((1, 1, 1, 1), (1, 1, 1, 1), (1, 1), "SAME", (1, 1), MM),
+    ((1, 14, 14, 7), (7, 7, 7, 10), (2, 2), "SAME", (1, 1), MM),
+]
+
+
+def _check(pkg, oracle, table, x, f, mm, strides, padding, dil, fast=False, depthwise=False):
+    y, acc = gpu_util.run_op(pkg, table, x, f, mm, strides, padding, dil, depthwise=depthwise)
+    if depthwise:
+        rc, y_ref, acc_ref = oracle.depthwise_conv2d(table, x, f, *mm, strides=strides, padding=padding, dilations=dil)
+    elif fast:
+        rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding, dilations=dil, threads=16)
+    else:
+        rc, y_ref, acc_ref = oracle.conv2d(table, x, f, *mm, strides=strides, padding=padding, dilations=dil)
+    assert rc == 0
+    assert acc.shape == acc_ref.shape and y.shape == y_ref.shape
+    assert np.array_equal(acc, acc_ref), "int32 accumulators differ"
+    # The reference accumulates float(table entry) in fp32 (approx_nn_conv_kernels.cpp:235,246): exact while
+    # the running sum stays below 2^24, rounded at every step beyond.  The HIP path converts the exact int32
+    # sum once.  Above 2^24 the reference's own rounding, at most K * 2^-24 of the sum, is allowed on top.
+    slack = 0.0
+    if not fast and not depthwise and acc_ref.size and int(acc_ref.max()) > (1 << 24):
+        K = f.shape[0] * f.shape[1] * f.shape[2]
+        qp = oracle.quant_props(*mm)
+        slack = K * 2.0 ** -24 * float(acc_ref.max()) * abs(float(qp.s1xs2)) / float(np.max(np.abs(y_ref)))
+        rc2, y_int, _ = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding, dilations=dil, threads=16)
+        assert rc2 == 0 and refimpl.linf_rel(y, y_int) <= TOL      # same integer sums, one conversion: tight
+    assert refimpl.linf_rel(y, y_ref) <= TOL + slack
+    return y, acc
+
+
+@pytest.mark.parametrize("case", SMALL, ids=[str(i) for i in range(len(SMALL))])
+@pytest.mark.parametrize("tname", ["random", "asymmetric", "exact"])
+def test_dense_vs_reference_order_oracle(pkg, oracle, case, tname):
+    xs, fs, strides, padding, dil, mm = case
+    table = {"random": pkg.synth.table_random(3), "asymmetric": pkg.synth.table_asymmetric(),
+             "exact": pkg.synth.table_exact()}[tname]
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, mm, seed=len(str(case)) + len(tname))
+    _check(pkg, oracle, table, x, f, mm, strides, padding, dil)
+
+
+def test_config1_both_tables_and_committed_vectors(pkg, oracle, golden_dir):
+    z = np.load(os.path.join(golden_dir, "config1_oracle.npz"))
+    mm = tuple(float(v) for v in z["minmax"])
+    for tname, table in (("exact", pkg.synth.table_exact()), ("noisy", pkg.synth.table_noisy(seed=7))):
+        y, acc = gpu_util.run_op(pkg, table, z["x"], z["f"], mm)
+        assert np.array_equal(acc, z["acc_" + tname])
+        assert refimpl.linf_rel(y, z["y_" + tname]) <= TOL
+
+
+def test_reference_tables_from_files(pkg, oracle, golden_dir):
+    """Every committed reference table, loaded through the file entry point (the op's mul_map_file attr)."""
+    case = pkg.synth.config1(seed=2)
+    for name in sorted(os.listdir(os.path.join(golden_dir, "tables"))):
+        path = os.path.join(golden_dir, "tables", name)
+        table_np = oracle.table_load(path)
+        xd = torch.from_numpy(case["x"]).to(gpu_util.dev())
+        fd = torch.from_numpy(case["f"]).to(gpu_util.dev())
+        y = pkg.approx_conv2d_with_min_max_vars(xd, fd, *case["minmax"], [1, 1, 1, 1], 8, path, "SAME").cpu().numpy()
+        rc, y_ref, _ = oracle.conv2d_fast(table_np, case["x"], case["f"], *case["minmax"], threads=8)
+        assert rc == 0 and refimpl.linf_rel(y, y_ref) <= TOL, name
+
+
+def test_empty_mul_map_file_means_exact_products(pkg, oracle):
+    case = pkg.synth.config1(seed=3)
+    xd = torch.from_numpy(case["x"]).to(gpu_util.dev())
+    fd = torch.from_numpy(case["f"]).to(gpu_util.dev())
+    y = pkg.approx_conv2d_with_min_max_vars(xd, fd, *case["minmax"], [1, 1, 1, 1], 8, "", "SAME").cpu().numpy()
+    rc, y_ref, _ = oracle.conv2d_fast(oracle.table_exact(), case["x"], case["f"], *case["minmax"], threads=8)
+    assert refimpl.linf_rel(y, y_ref) <= TOL
+
+
+def test_the_reference_test_recipe(pkg, golden_dir):
+    """tf2/test/test_table_approx_conv_2d.py: rand[1,256,256,1] (*) rand[8,8,1,1], min/max 0/1, fake-quantized,
+    exact table file, SAME; compared with a library convolution.  Expected Linf ~3e-7 (tf2/README.md:30-31)."""
+    rng = np.random.default_rng(0)
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    x = fq(rng.random((1, 256, 256, 1), dtype=np.float32), 0.0, 1.0)
+    f = fq(rng.random((8, 8, 1, 1), dtype=np.float32), 0.0, 1.0)
+    xd, fd = torch.from_numpy(x).to(gpu_util.dev()), torch.from_numpy(f).to(gpu_util.dev())
+    y = pkg.approx_conv2d_with_min_max_vars(xd, fd, 0.0, 1.0, 0.0, 1.0, [1, 1, 1, 1], 8,
+                                            os.path.join(golden_dir, "tables", "test_mul_table.bin"), "SAME")
+    ref = refimpl.torch_conv2d_f64(x, f)
+    assert refimpl.linf_rel(y.cpu().numpy(), ref) < 2e-6
+
+
+MEDIUM = [
+    ((128, 32, 32, 3), (3, 3, 3, 16), (1, 1)),      # config 2 stem
+    ((32, 32, 32, 16), (3, 3, 16, 16), (1, 1)),     # config 2 stage 1 (quarter batch)
+    ((32, 32, 32, 16), (3, 3, 16, 32), (2, 2)),     # config 2 downsample
+    ((32, 16, 16, 32), (3, 3, 32, 64), (2, 2)),
+    ((16, 8, 8, 64), (3, 3, 64, 64), (1, 1)),
+    ((2, 56, 56, 64), (3, 3, 64, 64), (1, 1)),      # north-star layer at batch 2
+    ((1, 28, 28, 128), (1, 1, 128, 256), (1, 1)),   # 1x1 expand
+    ((1, 30, 30, 24), (7, 7, 24, 64), (2, 2)),      # 7x7/2 stem shape
+]
+
+
+@pytest.mark.parametrize("case", MEDIUM, ids=[str(i) for i in range(len(MEDIUM))])
+def test_dense_medium_vs_oracle(pkg, oracle, case):
+    xs, fs, strides = case
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=xs[0] + fs[3], codes="halfnormal")
+    _check(pkg, oracle, pkg.synth.table_uniform_error(11), x, f, MM, strides, "SAME", (1, 1), fast=True)
+
+
+def test_he_normal_weights_with_tensor_minmax(pkg, oracle):
+    """The Keras wrapper's policy: min/max are the tensors' own extrema (fake_approx_convolutional.py:233-242)."""
+    rng = np.random.default_rng(5)
+    x = rng.uniform(0, 1, (4, 16, 16, 16)).astype(np.float32)
+    in_min, in_max = float(x.min()), float(x.max())
+    x = pkg.fake_quant.fake_quant_with_min_max_vars(x, in_min, in_max)
+    f, f_min, f_max = pkg.synth.he_normal_filter((3, 3, 16, 32), seed=6)
+    _check(pkg, oracle, pkg.synth.table_noisy(7), x, f, (in_min, in_max, f_min, f_max), (1, 1), "SAME", (1, 1), fast=True)
+
+
+def test_off_grid_inputs_quantize_like_the_reference(pkg, oracle):
+    """Inputs that were not fake-quantized (but lie inside the range) still go through the same
+    three-rounding quantize expression, so codes and sums stay bit-exact."""
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-0.99, 0.99, (2, 10, 10, 6)).astype(np.float32)
+    f = rng.uniform(-0.49, 0.49, (3, 3, 6, 12)).astype(np.float32)
+    _check(pkg, oracle, pkg.synth.table_random(4), x, f, MM, (1, 1), "SAME", (1, 1))
+
+
+def test_zero_range_tensors(pkg, oracle):
+    """min == max == 0 gives scale = inv_scale = offset = 0 (approx_ops_types.h:142-151): every code is 0."""
+    x = np.zeros((1, 6, 6, 4), np.float32)
+    f, _, _ = pkg.synth.he_normal_filter((3, 3, 4, 8), seed=1)
+    _check(pkg, oracle, pkg.synth.table_asymmetric(), x, f, (0.0, 0.0, -0.5, 0.5), (1, 1), "SAME", (1, 1))
+
+
+def test_empty_batch_returns_empty_output(pkg):
+    op = pkg.ApproxConv2DWithMinMaxVars([1, 1, 1, 1], 8, pkg.synth.table_exact(), "SAME")
+    x = torch.zeros((0, 8, 8, 4), device=gpu_util.dev())
+    f = torch.zeros((3, 3, 4, 8), device=gpu_util.dev())
+    assert tuple(op(x, f, *MM).shape) == (0, 8, 8, 8)
+
+
+def test_quantize_entry_point(pkg, oracle):
+    from tf_approximate_amd import ops
+    rng = np.random.default_rng(3)
+    for vmin, vmax in [(-1.0, 1.0), (0.0, 6.0), (-0.3, 0.3), (-0.017, 0.093)]:
+        span = vmax - vmin
+        v = rng.uniform(vmin - 0.2 * span, vmax + 0.2 * span, 200000).astype(np.float32)   # also out of range: clamps
+        nmin, _, scale = oracle.nudge(vmin, vmax)
+        grid = pkg.fake_quant.grid_value(np.arange(256), vmin, vmax)
+        v = np.concatenate([v, grid, np.zeros(3, np.float32), np.array([np.nan, np.inf, -np.inf], np.float32)])
+        codes = ops.quantize(torch.from_numpy(v).to(gpu_util.dev()), vmin, vmax).cpu().numpy()
+        qp = oracle.quant_props(vmin, vmax, 0.0, 0.0)
+        want = oracle.quantize(v, qp.in_offset, qp.in_inv_scale)
+        finite = np.isfinite(v)
+        assert np.array_equal(codes[finite], want[finite])
+        assert codes[-3] == 0 and codes[-2] == 255 and codes[-1] == 0      # NaN -> 0, +inf -> 255, -inf -> 0
+
+
+def test_codes_entry_point(pkg, oracle):
+    from tf_approximate_amd import ops
+    rng = np.random.default_rng(8)
+    table_np = pkg.synth.table_random(21)
+    table = pkg.TruthTable(table_np)
+    for xs, fs, strides, padding, zp in [((2, 9, 8, 5), (3, 3, 5, 11), (1, 1), "SAME", 17),
+                                         ((1, 13, 13, 32), (3, 3, 32, 64), (2, 2), "SAME", 0),
+                                         ((3, 6, 6, 16), (1, 1, 16, 48), (1, 1), "VALID", 255)]:
+        qa = rng.integers(0, 256, xs).astype(np.uint8)
+        qb = rng.integers(0, 256, fs).astype(np.uint8)
+        acc = ops.conv2d_codes_acc_i32(table, torch.from_numpy(qa).to(gpu_util.dev()),
+                                       torch.from_numpy(qb).to(gpu_util.dev()), zp,
+                                       (1, strides[0], strides[1], 1), padding).cpu().numpy()
+        patches = refimpl.gather_patches(qa, zp, fs[0], fs[1], strides, padding, (1, 1))
+        n, oh, ow = patches.shape[:3]
+        want = oracle.lut_gemm_codes(table_np, patches.reshape(n * oh * ow, -1), qb.reshape(-1, fs[3]))
+        assert np.array_equal(acc.reshape(n * oh * ow, fs[3]), want)
+
+
+DEPTHWISE = [
+    ((2, 10, 10, 12), (3, 3, 12, 1), (1, 1), "SAME"),
+    ((2, 11, 9, 70), (3, 3, 70, 1), (2, 2), "SAME"),
+    ((1, 8, 8, 3), (5, 5, 3, 1), (1, 1), "VALID"),
+    ((2, 28, 28, 192), (3, 3, 192, 1), (1, 1), "SAME"),   # MobileNetV2-style block at reduced size
+    ((2, 28, 28, 192), (3, 3, 192, 1), (2, 2), "SAME"),
+]
+
+
+@pytest.mark.parametrize("case", DEPTHWISE, ids=[str(i) for i in range(len(DEPTHWISE))])
+@pytest.mark.parametrize("k", [2, 4])
+def test_depthwise_vs_oracle(pkg, oracle, case, k):
+    xs, fs, strides, padding = case
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=k + xs[3])
+    _check(pkg, oracle, pkg.synth.table_truncated(k), x, f, MM, strides, padding, (1, 1), depthwise=True)
+
+
+def test_inverted_residual_block(pkg, oracle):
+    """1x1 expand (x6) -> depthwise 3x3 -> 1x1 project, each layer against the oracle."""
+    rng = np.random.default_rng(2)
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    x = fq(rng.uniform(-1, 1, (2, 14, 14, 32)).astype(np.float32), -1.0, 1.0)
+    layers = [((1, 1, 32, 192), False, (1, 1)), ((3, 3, 192, 1), True, (2, 2)), ((1, 1, 192, 32), False, (1, 1))]
+    for i, (fs, dw, strides) in enumerate(layers):
+        f, f_min, f_max = pkg.synth.he_normal_filter(fs, seed=40 + i)
+        in_min, in_max = float(x.min()), float(x.max())
+        x = fq(x, in_min, in_max)
+        table = pkg.synth.table_truncated(2 if i % 2 else 4)
+        y, _ = _check(pkg, oracle, table, x, f, (in_min, in_max, f_min, f_max), strides, "SAME", (1, 1),
+                      fast=True, depthwise=dw)
+        x = np.maximum(y, 0.0)
+
+
+def test_error_paths_on_device(pkg):
+    op = pkg.ApproxConv2DWithMinMaxVars([1, 1, 1, 1], 8, pkg.synth.table_exact(), "SAME")
+    x = torch.zeros((1, 8, 8, 4), device=gpu_util.dev())
+    with pytest.raises(pkg.UnimplementedError, match="grouped convolutions"):
+        op(x, torch.zeros((3, 3, 2, 8), device=gpu_util.dev()), *MM)
+    with pytest.raises(pkg.InvalidArgumentError, match="evenly divisible"):
+        op(x, torch.zeros((3, 3, 3, 8), device=gpu_util.dev()), *MM)
+    with pytest.raises(pkg.UnimplementedError, match="float32"):
+        op(x.half(), torch.zeros((3, 3, 4, 8), device=gpu_util.dev()).half(), *MM)
+    with pytest.raises(pkg.InvalidArgumentError):
+        op(x.cpu(), torch.zeros((3, 3, 4, 8)), *MM)
+    ex = pkg.ApproxConv2DWithMinMaxVars([1, 1, 1, 1], 8, pkg.synth.table_exact(), "EXPLICIT",
+                                        explicit_paddings=[0, 0, 1, 1, 1, 1, 0, 0])
+    with pytest.raises(pkg.UnimplementedError, match="Explicit padding is not implemented"):
+        ex(x, torch.zeros((3, 3, 4, 8), device=gpu_util.dev()), *MM)
+    with pytest.raises(pkg.InvalidArgumentError, match="Couldn't read the lookup table"):
+        pkg.TruthTable("/nonexistent/table.bin")
+    # a workspace that is too small is refused before anything is launched
+    from tf_approximate_amd import _lib, ops
+    lib = _lib.load()
+    desc = ops.make_desc((1, 8, 8, 4), (3, 3, 4, 8), (1, 1, 1, 1), "SAME")
+    f = torch.zeros((3, 3, 4, 8), device=gpu_util.dev())
+    y = torch.zeros((1, 8, 8, 8), device=gpu_util.dev())
+    ws = torch.zeros(256, dtype=torch.uint8, device=gpu_util.dev())
+    rc = lib.axc_conv2d_minmax(op.table.handle, ctypes.byref(desc), x.data_ptr(), f.data_ptr(), -1.0, 1.0, -0.5, 0.5,
+                               y.data_ptr(), ws.data_ptr(), 256, None)
+    assert rc == 1 and b"workspace too small" in lib.axc_last_error()
+
+
+def test_non_default_stream(pkg, oracle):
+    case = pkg.synth.config1(seed=4)
+    table = pkg.synth.table_noisy(7)
+    op = pkg.ApproxConv2DWithMinMaxVars([1, 1, 1, 1], 8, table, "SAME")
+    s = torch.cuda.Stream(device=gpu_util.dev())
+    xd = torch.from_numpy(case["x"]).to(gpu_util.dev())
+    fd = torch.from_numpy(case["f"]).to(gpu_util.dev())
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        y = op(xd, fd, *case["minmax"])
+    s.synchronize()
+    rc, y_ref, _ = oracle.conv2d_fast(table, case["x"], case["f"], *case["minmax"], threads=8)
+    assert refimpl.linf_rel(y.cpu().numpy(), y_ref) <= TOL

@@ -1,0 +1,183 @@
+"""CPU-side checks of the product's host code: the C-ABI library loads and exports every symbol the
+header declares, and its geometry / quantization-parameter / argument-checking logic agrees with the
+oracle and with the reference's error behaviour.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib(pkg):
+    from tf_approximate_amd import _lib
+    return _lib.load()
+
+
+@pytest.fixture(scope="module")
+def ops(pkg):
+    from tf_approximate_amd import ops
+    return ops
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "axconv.h")).read()
+    declared = set(re.findall(r"\b(axc_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 20
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+    from tf_approximate_amd import _lib
+    assert declared == {n for n, _, _ in _lib.SYMBOLS}
+
+
+def test_status_strings(lib):
+    assert lib.axc_status_string(0) == b"OK"
+    assert lib.axc_status_string(1) == b"INVALID_ARGUMENT"
+    assert lib.axc_status_string(2) == b"UNIMPLEMENTED"
+    assert lib.axc_status_string(3) == b"RUNTIME_ERROR"
+
+
+@pytest.mark.parametrize("mm", [(-1.0, 1.0, -0.3, 0.3), (0.0, 1.0, -0.5, 0.5), (0.0, 6.0, -0.017, 0.093),
+                                (-2.5, 0.0, 0.0, 0.0), (0.0, 0.0, -1.0, 2.0)])
+def test_quant_props_bit_equal_to_oracle(ops, oracle, mm):
+    a = ops.quant_props(*mm)
+    b = oracle.quant_props(*mm)
+    pairs = [(a.input_scale, b.in_scale), (a.input_inv_scale, b.in_inv_scale), (a.input_offset, b.in_offset),
+             (a.filter_scale, b.f_scale), (a.filter_inv_scale, b.f_inv_scale), (a.filter_offset, b.f_offset),
+             (a.s1xs2, b.s1xs2), (a.m1, b.m1), (a.m2, b.m2), (a.m1xm2, b.m1xm2)]
+    for x, y in pairs:
+        assert np.float32(x).tobytes() == np.float32(y).tobytes()
+    zc = oracle.quantize(np.zeros(1, np.float32), b.in_offset, b.in_inv_scale)[0]
+    assert a.input_zero_code == zc
+
+
+def test_geometry_matches_oracle(ops, oracle):
+    rng = np.random.default_rng(0)
+    for _ in range(300):
+        h, w = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        kh, kw = int(rng.integers(1, 9)), int(rng.integers(1, 9))
+        s = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        d = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        padding = "SAME" if rng.integers(0, 2) else "VALID"
+        rc, g = oracle.geometry((2, h, w, 3), (kh, kw, 3, 5), s, padding, d)
+        desc = ops.make_desc((2, h, w, 3), (kh, kw, 3, 5), (1, s[0], s[1], 1), padding, (), "NHWC", (1, d[0], d[1], 1))
+        if rc != 0:
+            with pytest.raises(ops.InvalidArgumentError):
+                ops.conv2d_geometry(desc)
+            continue
+        dims = ops.conv2d_geometry(desc)
+        assert (dims.out_rows, dims.out_cols) == (g.out_rows, g.out_cols)
+        assert (dims.pad_rows_before, dims.pad_cols_before) == (g.pad_rows_before, g.pad_cols_before)
+        assert (dims.pad_rows_after, dims.pad_cols_after) == (g.pad_rows_after, g.pad_cols_after)
+
+
+def test_nchw_strides_are_read_in_format_order(ops):
+    desc = ops.make_desc((2, 3, 10, 12), (3, 3, 3, 5), (1, 1, 2, 2), "SAME", (), "NCHW", (1, 1, 1, 1))
+    dims = ops.conv2d_geometry(desc)
+    assert (dims.batch, dims.in_depth, dims.input_rows, dims.input_cols) == (2, 3, 10, 12)
+    assert (dims.out_rows, dims.out_cols) == (5, 6)
+
+
+def _ws(lib, desc, depthwise=False):
+    n = ctypes.c_size_t()
+    fn = lib.axc_depthwise_conv2d_workspace_bytes if depthwise else lib.axc_conv2d_workspace_bytes
+    return fn(ctypes.byref(desc), ctypes.byref(n)), n.value
+
+
+def test_attr_errors_mirror_the_reference(ops, lib):
+    """Messages of InitApproxConv2DParameters / the launchers (tf2/src/approx_nn_conv_ops.cpp:120,162,224,231,287-303)."""
+    ok = dict(input_shape=(1, 8, 8, 4), filter_shape=(3, 3, 4, 8), strides=(1, 1, 1, 1), padding="SAME")
+
+    def geom(**kw):
+        a = dict(ok)
+        a.update(kw)
+        return ops.conv2d_geometry(ops.make_desc(**a))
+
+    with pytest.raises(ops.InvalidArgumentError, match="strides in the batch and depth"):
+        geom(strides=(2, 1, 1, 1))
+    with pytest.raises(ops.InvalidArgumentError, match="strides in the batch and depth"):
+        geom(strides=(1, 1, 1, 2))
+    with pytest.raises(ops.InvalidArgumentError, match="strides should be larger than 0"):
+        geom(strides=(1, 0, 1, 1))
+    with pytest.raises(ops.InvalidArgumentError, match="dilations in the batch and depth"):
+        geom(dilations=(1, 1, 1, 2))
+    with pytest.raises(ops.InvalidArgumentError, match="Dilated rates should be larger than 0"):
+        geom(dilations=(1, 0, 1, 1))
+    with pytest.raises(ops.InvalidArgumentError, match="4 dimensions"):
+        geom(strides=(1, 1))
+    with pytest.raises(ops.InvalidArgumentError, match="must be 4-dimensional"):
+        geom(input_shape=(8, 8, 4))
+    with pytest.raises(ops.InvalidArgumentError, match="evenly divisible"):
+        geom(filter_shape=(3, 3, 3, 8))
+    with pytest.raises(ops.InvalidArgumentError, match="Invalid data format"):
+        geom(data_format="NHCW")
+
+    def ws(**kw):
+        a = dict(ok)
+        a.update(kw)
+        rc, _ = _ws(lib, ops.make_desc(**a))
+        return rc, lib.axc_last_error().decode()
+
+    rc, msg = ws(padding="EXPLICIT", explicit_paddings=(0, 0, 1, 1, 1, 1, 0, 0))
+    assert rc == 2 and msg == "Explicit padding is not implemented."
+    rc, msg = ws(filter_shape=(3, 3, 2, 8))
+    assert rc == 2 and "grouped convolutions" in msg
+    rc, msg = ws(input_shape=(1, 4, 8, 8), data_format="NCHW")
+    assert rc == 2 and "only supports NHWC" in msg
+    rc, msg = ws(num_bits=4)
+    assert rc == 1 and "num_bits" in msg
+    rc, msg = ws(input_shape=(1, 200, 200, 64), filter_shape=(30, 30, 64, 8), padding="VALID")
+    assert rc == 1 and "patch length" in msg            # int32 accumulator bound, K >= 32768
+    rc, msg = ws(input_shape=(1, 2100, 2100, 1), filter_shape=(2049, 2049, 1, 1), padding="VALID")
+    assert rc == 1 and msg == "ApproxConv2DOp: Patch too large for buffer"
+
+
+def test_workspace_sizes(ops, lib):
+    desc = ops.make_desc((64, 56, 56, 64), (3, 3, 64, 64), (1, 1, 1, 1), "SAME")
+    rc, n = _ws(lib, desc)
+    assert rc == 0
+    xq = 64 * 56 * 56 * 64            # one byte per activation
+    psum = 64 * 56 * 56 * 4
+    assert xq + psum < n < xq + psum + (1 << 20)
+    rc, n0 = _ws(lib, ops.make_desc((0, 56, 56, 64), (3, 3, 64, 64), (1, 1, 1, 1), "SAME"))
+    assert rc == 0 and n0 == 0        # empty output: nothing to do (approx_nn_conv_ops.cpp:449)
+    rc, nd = _ws(lib, ops.make_desc((2, 8, 8, 6), (3, 3, 6, 1), (1, 1, 1, 1), "SAME"), depthwise=True)
+    assert rc == 0 and nd >= 9 * 6 + 6 * 4
+    rc, _ = _ws(lib, ops.make_desc((2, 8, 8, 6), (3, 3, 6, 2), (1, 1, 1, 1), "SAME"), depthwise=True)
+    assert rc == 1
+
+
+def test_table_file_errors_need_no_gpu(lib, tmp_path):
+    """Short read / missing file -> InvalidArgument with the reference's text (approx_ops_types.h:213)."""
+    p = tmp_path / "short.bin"
+    p.write_bytes(b"\x01" * 4096)
+    h = ctypes.c_void_p()
+    assert lib.axc_table_create_from_file(str(p).encode(), 8, ctypes.byref(h)) == 1
+    assert lib.axc_last_error() == b"ApproxTF: Couldn't read the lookup table!"
+    assert lib.axc_table_create_from_file(str(tmp_path / "none.bin").encode(), 8, ctypes.byref(h)) == 1
+    assert lib.axc_table_create_from_file(b"", 7, ctypes.byref(h)) == 1
+    assert b"num_bits" in lib.axc_last_error()
+
+
+def test_synthetic_tables(pkg):
+    s = pkg.synth
+    assert s.table_exact()[3 * 256 + 5] == 15
+    for t in (s.table_noisy(7), s.table_truncated(2), s.table_truncated(4), s.table_uniform_error(11),
+              s.table_random(13), s.table_asymmetric()):
+        assert t.dtype == np.uint16 and t.shape == (65536,)
+    assert np.array_equal(s.table_noisy(7), s.table_noisy(7))
+    t4 = s.table_truncated(4).reshape(256, 256).astype(np.int64)
+    ab = np.arange(256)[:, None] * np.arange(256)[None, :]
+    assert np.array_equal(t4, ab - ab % 16)
+    assert s.table_asymmetric().reshape(256, 256)[0].min() > 0
+
+
+def test_missing_library_fails_loudly(pkg, monkeypatch):
+    from tf_approximate_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libaxconv_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.load()

@@ -41,7 +41,7 @@ struct DenseParams {
     ConvGeom g;
     DensePlan plan;
     const uint32_t *xq;     // [N][H][C4][W] dwords of 4 row-permuted activation codes
-    const float *chsum;     // [N][H][W] sum over channels of the raw input (float epilogue only)
+    const float *psum;      // [M] sum of the raw input over each output pixel's patch (float epilogue only)
     const uint16_t *wq;     // [n_col_tiles][fills][64] packed filter codes (kNullWeight = none)
     const float *fsum;      // [Co] sum over (h, w, c) of the raw filter
     const uint16_t *tableT; // [256 filter code][256 input code]
@@ -81,6 +81,7 @@ __device__ inline uint32_t quantize_code(float v, float offset, float inv_scale)
 // ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
 hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
                                     uint32_t *xq, float *chsum, hipStream_t stream);
+hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream);
 hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t *xq, hipStream_t stream);
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
                               const DensePlan &plan, float offset, float inv_scale,

@@ -229,19 +229,8 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
             if (!rvalid[r])
                 continue;
             const int64_t m = row0 + (int64_t)(r * kWaves + wave) * 64 + lane;
-            float psum = 0.0f;
-            if (!OUT_I32) {
-                // patch sum = sum over taps of the per-pixel channel sums (0 outside the image)
-                const int n = (int)(m / ((int64_t)g.OH * g.OW));
-                const int ih0 = hw0[r] >> 16;
-                const int iw0 = (int)(int16_t)(hw0[r] & 0xffff);
-                for (int kh = 0; kh < g.KH; ++kh)
-                    for (int kw = 0; kw < g.KW; ++kw) {
-                        const int ih = ih0 + kh * g.dh, iw = iw0 + kw * g.dw;
-                        if ((unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
-                            psum = __fadd_rn(psum, p.chsum[((int64_t)n * g.H + ih) * g.W + iw]);
-                    }
-            }
+            // patch sum of the raw input in the reference's order (tap-major, channels ascending)
+            const float psum = OUT_I32 ? 0.0f : p.psum[m];
             const float t1 = __fmul_rn(p.m2, psum);
 #pragma unroll
             for (int set = 0; set < SETS; ++set) {

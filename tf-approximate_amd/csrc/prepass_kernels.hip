@@ -39,6 +39,49 @@ __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__r
         chsum[pix] = sum;
 }
 
+// Patch sums (the outCoeffs of ApproxConvIm2ColKernel, tf2/src/approx_nn_conv_kernels.cpp:294): for each
+// output pixel the fp32 sum of the raw input over its patch, accumulated strictly in the reference's order
+// (kh, kw, c ascending; taps outside the image add 0.0f, which leaves the sum unchanged).  fp32 addition is
+// not associative and this sum is multiplied by the filter offset in the epilogue, so any other order
+// shows up in the output at the 1e-4 level for inputs with a large mean.  One thread per output pixel.
+__global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict__ x, ConvGeom g,
+                                                          float *__restrict__ psum)
+{
+    const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= g.M)
+        return;
+    const int n = (int)(m / ((int64_t)g.OH * g.OW));
+    const int rem = (int)(m - (int64_t)n * g.OH * g.OW);
+    const int oh = rem / g.OW, ow = rem - oh * g.OW;
+    const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
+    float s = 0.0f;
+    for (int kh = 0; kh < g.KH; ++kh) {
+        const int ih = ih0 + kh * g.dh;
+        if ((unsigned)ih >= (unsigned)g.H)
+            continue;
+        for (int kw = 0; kw < g.KW; ++kw) {
+            const int iw = iw0 + kw * g.dw;
+            if ((unsigned)iw >= (unsigned)g.W)
+                continue;
+            const float *src = x + (((int64_t)n * g.H + ih) * g.W + iw) * g.C;
+            if ((g.C & 3) == 0) {
+                const float4 *src4 = reinterpret_cast<const float4 *>(src);
+                for (int c4 = 0; c4 < g.C / 4; ++c4) {
+                    const float4 v = src4[c4];
+                    s = __fadd_rn(s, v.x);
+                    s = __fadd_rn(s, v.y);
+                    s = __fadd_rn(s, v.z);
+                    s = __fadd_rn(s, v.w);
+                }
+            } else {
+                for (int c = 0; c < g.C; ++c)
+                    s = __fadd_rn(s, src[c]);
+            }
+        }
+    }
+    psum[m] = s;
+}
+
 // Same relayout for caller-supplied codes (uint8 NHWC).
 __global__ void __launch_bounds__(256) codes_relayout_kernel(const uint8_t *__restrict__ codes, int64_t pixels,
                                                               int W, int C, int C4, uint32_t *__restrict__ xq)
@@ -145,6 +188,12 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float off
     const int64_t pixels = (int64_t)g.N * g.H * g.W;
     hipLaunchKernelGGL(quantize_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, x, pixels,
                        g.H, g.W, g.C, g.C4, offset, inv_scale, xq, chsum);
+    return hipGetLastError();
+}
+
+hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream)
+{
+    hipLaunchKernelGGL(patch_sums_kernel, dim3(blocks_for(g.M, 256)), dim3(256), 0, stream, x, g, psum);
     return hipGetLastError();
 }
 
