@@ -329,9 +329,7 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
     DenseWorkspace w;
     size_t off = 0;
     w.xq_off = off; off += align_up((size_t)g.N * g.H * g.C4 * g.W * 4);
-    // patch sums: one float per output pixel (for 1x1 stride-1 filters the per-pixel channel sums)
-    const size_t psum_elems = (size_t)g.M > (size_t)g.N * g.H * g.W ? (size_t)g.M : (size_t)g.N * g.H * g.W;
-    w.psum_off = off; off += align_up(psum_elems * 4);
+    w.psum_off = off; off += align_up((size_t)g.M * 4); // patch sums: one float per output pixel
     w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
     w.fsum_off = off; off += align_up((size_t)g.Co * 4);
     w.total = off;
@@ -414,8 +412,6 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     char *ws = static_cast<char *>(workspace);
     uint32_t *xq = reinterpret_cast<uint32_t *>(ws + pd.ws.xq_off);
     float *psum = reinterpret_cast<float *>(ws + pd.ws.psum_off);
-    // A 1x1 stride-1 filter's patch is the pixel itself: the pre-pass's channel sums are the patch sums.
-    const bool pixel_is_patch = g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0;
     uint16_t *wq = reinterpret_cast<uint16_t *>(ws + pd.ws.wq_off);
     float *fsum = reinterpret_cast<float *>(ws + pd.ws.fsum_off);
 
@@ -424,10 +420,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         AXC_HIP(launch_codes_relayout(input_codes, g, xq, stream));
     } else {
         ProfScope ps("quantize_relayout", stream);
-        AXC_HIP(launch_quantize_relayout(input, g, qp.input_offset, qp.input_inv_scale, xq,
-                                         (out_f && pixel_is_patch) ? psum : nullptr, stream));
+        AXC_HIP(launch_quantize_relayout(input, g, qp.input_offset, qp.input_inv_scale, xq, nullptr, stream));
     }
-    if (out_f && !codes_mode && !pixel_is_patch) {
+    if (out_f && !codes_mode) {
         ProfScope ps("patch_sums", stream);
         AXC_HIP(launch_patch_sums(input, g, psum, stream));
     }

@@ -15,6 +15,7 @@
 // Restates, as one fused kernel, what the reference does in ApproxConvIm2ColKernel +
 // ApproxConvGEMMKernel (tf2/src/approx_nn_conv_kernels.cpp:215-296) per chunk.
 #include "axconv_internal.h"
+#include "lookup_asm.inc"
 
 namespace axc {
 
@@ -22,6 +23,19 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 extern __shared__ __align__(16) unsigned char lds[];
+
+// Four table-row reads in flight, then one wait: the compiler would serialize them.
+__device__ __forceinline__ void lds_read4_b64(uint64_t (&v)[4], const uint32_t (&addr)[4])
+{
+    asm volatile("ds_read_b64 %0, %4\n\t"
+                 "ds_read_b64 %1, %5\n\t"
+                 "ds_read_b64 %2, %6\n\t"
+                 "ds_read_b64 %3, %7\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
+                 : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3])
+                 : "memory");
+}
 
 template <int NT, bool OUT_I32>
 __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const DenseParams p)
@@ -35,7 +49,7 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
     const ConvGeom &g = p.g;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: row activity branches on SGPRs
 
     // ---- stage the truth table (once per workgroup; the workgroup is persistent) ----
     {
@@ -71,6 +85,7 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
     const int taps = g.KH * g.KW;
     const int ntiles = p.plan.n_row_tiles * p.plan.n_col_tiles;
     const int fills = p.plan.fills;
+    const int rowstep = g.C4 * g.W; // dwords between input rows in xq
 
     for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int ct = tile % p.plan.n_col_tiles;
@@ -79,7 +94,7 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
         const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
 
         // ---- per-pixel geometry ----
-        int32_t nbase[R];  // dword index of (n, 0, 0, 0) in xq
+        int32_t pbase[R];  // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
         int hw0[R];        // (ih0 << 16) | (iw0 & 0xffff): input coordinates of tap (0, 0)
         bool rvalid[R];    // this lane's pixel exists
         bool ractive[R];   // some lane of this wavefront has a pixel (wave-uniform)
@@ -94,8 +109,9 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
             const int rem = (int)(mm - (int64_t)n * g.OH * g.OW);
             const int oh = rem / g.OW;
             const int ow = rem - oh * g.OW;
-            nbase[r] = n * g.H * g.C4 * g.W;
-            hw0[r] = ((oh * g.sh - g.ph) << 16) | ((ow * g.sw - g.pw) & 0xffff);
+            const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
+            pbase[r] = (n * g.H + ih0) * rowstep + iw0;
+            hw0[r] = (ih0 << 16) | (iw0 & 0xffff);
         }
 
         int32_t acc[R][NT];
@@ -105,122 +121,154 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
             for (int j = 0; j < NT; ++j)
                 acc[r][j] = 0;
 
-        const uint16_t *wq_tile = p.wq + (size_t)ct * fills * 64;
+        const uint16_t *wq_tile = p.wq + (size_t)ct * fills * 64 + jq * 4;
 
-        // ---- software pipeline: the loads of the next channel quad / next fill are issued
-        //      before the current fill's LDS work ----
-        int32_t base_n[R]; // dword index of the next quad to load, valid if inb_n
-        bool inb_n[R];
+        // ---- load cursor: (tap, quad) of the activation dwords to fetch next ----
         int tap_n = 0, q_n = 0, kh_n = 0, kw_n = 0;
+        bool inb_n[R];
+        int32_t idx_n[R];
         auto tap_setup = [&]() {
+            const int dh = kh_n * g.dh, dw = kw_n * g.dw;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int ih = (hw0[r] >> 16) + kh_n * g.dh;
-                const int iw = (int)(int16_t)(hw0[r] & 0xffff) + kw_n * g.dw;
+                const int ih = (hw0[r] >> 16) + dh;
+                const int iw = (int)(int16_t)(hw0[r] & 0xffff) + dw;
                 inb_n[r] = rvalid[r] && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-                base_n[r] = nbase[r] + ih * g.C4 * g.W + iw;
+                idx_n[r] = inb_n[r] ? pbase[r] + dh * rowstep + dw : 0;
             }
         };
         uint32_t a4n[R];
         auto issue_act_loads = [&]() {
+            // unconditional loads (index 0 when outside the image) keep the number of outstanding
+            // loads static, so waits on older loads do not have to drain these
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                a4n[r] = inb_n[r] ? p.xq[base_n[r] + q_n * g.W] : p.zp4;
+            for (int r = 0; r < R; ++r) {
+                const uint32_t v = p.xq[idx_n[r] + (inb_n[r] ? q_n * g.W : 0)];
+                a4n[r] = inb_n[r] ? v : p.zp4;
+            }
         };
+        auto advance_cursor = [&]() {
+            if (++q_n == g.C4) {
+                q_n = 0;
+                ++tap_n;
+                if (++kw_n == g.KW) { kw_n = 0; ++kh_n; }
+                if (tap_n < taps)
+                    tap_setup();
+            }
+        };
+
+        // derive phase, split so the table-row reads can run before the barrier that frees the
+        // expanded area and only the four writes sit between the two barriers
+        u32x2 o[4];
+        auto derive_read = [&](const u32x2 wc) {
+            const uint32_t code[4] = {wc.x & 0xffffu, wc.x >> 16, wc.y & 0xffffu, wc.y >> 16};
+            uint32_t addr[4];
+            bool none[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                none[i] = code[i] == kNullWeight;
+                addr[i] = (none[i] ? 0u : code[i]) * 512u + rd_off;
+            }
+            uint64_t v[4];
+            lds_read4_b64(v, addr);
+            uint32_t x[4], y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                x[i] = none[i] ? 0u : (uint32_t)v[i];
+                y[i] = none[i] ? 0u : (uint32_t)(v[i] >> 32);
+            }
+            o[0].x = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
+            o[0].y = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
+            o[1].x = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
+            o[1].y = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
+            o[2].x = __builtin_amdgcn_perm(y[1], y[0], 0x05040100u);
+            o[2].y = __builtin_amdgcn_perm(y[3], y[2], 0x05040100u);
+            o[3].x = __builtin_amdgcn_perm(y[1], y[0], 0x07060302u);
+            o[3].y = __builtin_amdgcn_perm(y[3], y[2], 0x07060302u);
+        };
+        auto derive_write = [&]() {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<u32x2 *>(lds + wr_off + (uint32_t)i * (64u * 128u)) = o[i];
+        };
+
+        // ---- prologue: activations of quad 0, weights of fill 0 -> expanded rows of fill 0 ----
+        uint32_t a4[R];
         tap_setup();
         issue_act_loads();
-        u32x2 wn = *reinterpret_cast<const u32x2 *>(wq_tile + jq * 4);
+        u32x2 wn = *reinterpret_cast<const u32x2 *>(wq_tile);
+        __syncthreads(); // table staged / previous tile's lookups done
+        derive_read(wn);
+        derive_write();
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            a4[r] = a4n[r];
+        advance_cursor();
+        if (tap_n < taps)
+            issue_act_loads();
+        if (fills > 1)
+            wn = *reinterpret_cast<const u32x2 *>(wq_tile + 64);
 
-        int fill = 0;
-        for (int tap = 0; tap < taps; ++tap) {
-            for (int q = 0; q < g.C4; ++q) {
-                uint32_t a4[R];
+        int sub = 0;
+        for (int fill = 0; fill < fills; ++fill) {
+            // ---- lookups of this fill ----
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (!ractive[r])
+                    continue;
+                // row offsets (128 B per activation code) of the channels of this fill
+                uint32_t ax = 0, ay = 0;
+                if (KS == 1) {
+                    ax = ((a4[r] >> (8 * sub)) & 0xffu) << 7;
+                } else if (KS == 2) {
+                    ax = ((a4[r] >> (16 * sub)) & 0xffu) << 7;
+                    ay = ((a4[r] >> (16 * sub + 8)) & 0xffu) << 7;
+                } else {
+                    ax = __builtin_amdgcn_alignbit(a4[r], a4[r], rot_kk0);
+                    ay = __builtin_amdgcn_alignbit(ax, ax, rot_p0);
+                }
+                uint32_t ad[8];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    uint32_t aoff;
+                    if (KS == 1)
+                        aoff = ax;
+                    else if (KS == 2)
+                        aoff = kk_hi[s] ? ay : ax;
+                    else
+                        aoff = ((((s & 1) ? ay : ax) >> (8 * (s >> 1))) & 0xffu) << 7;
+                    ad[s] = aoff + choff[s];
+                }
+                if constexpr (NT == 16) {
+                    LOOKUP_ROW_NT16(acc[r], ad);
+                } else if constexpr (NT == 32) {
+                    LOOKUP_ROW_NT32(acc[r], ad);
+                } else {
+                    LOOKUP_ROW_NT64(acc[r], ad);
+                }
+            }
+            if (fill + 1 == fills)
+                break;
+
+            // ---- expanded rows of the next fill ----
+            derive_read(wn);   // table-row reads + transposes overlap other wavefronts' lookups
+            __syncthreads();   // every wavefront is done reading the expanded rows of this fill
+            derive_write();
+            __syncthreads();
+
+            // ---- roll the pipeline: consume the prefetched registers, then issue the next loads ----
+            if (++sub == SUBS) {
+                sub = 0;
 #pragma unroll
                 for (int r = 0; r < R; ++r)
                     a4[r] = a4n[r];
-                // advance the load cursor and issue the next quad's loads
-                if (++q_n == g.C4) {
-                    q_n = 0;
-                    ++tap_n;
-                    if (++kw_n == g.KW) { kw_n = 0; ++kh_n; }
-                    if (tap_n < taps)
-                        tap_setup();
-                }
+                advance_cursor();
                 if (tap_n < taps)
                     issue_act_loads();
-
-#pragma unroll
-                for (int sub = 0; sub < SUBS; ++sub, ++fill) {
-                    const u32x2 wc = wn;
-                    if (fill + 1 < fills)
-                        wn = *reinterpret_cast<const u32x2 *>(wq_tile + (size_t)(fill + 1) * 64 + jq * 4);
-
-                    // ---- derive: expanded rows for this fill's 64 slots ----
-                    __syncthreads(); // previous fill's lookups (and the table staging) are done
-                    {
-                        uint32_t code[4] = {wc.x & 0xffffu, wc.x >> 16, wc.y & 0xffffu, wc.y >> 16};
-                        u32x2 v[4];
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const bool none = code[i] == kNullWeight;
-                            const uint32_t row = none ? 0u : code[i];
-                            v[i] = *reinterpret_cast<const u32x2 *>(lds + row * 512u + rd_off);
-                            if (none) { v[i].x = 0u; v[i].y = 0u; }
-                        }
-                        u32x2 o[4];
-                        o[0].x = __builtin_amdgcn_perm(v[1].x, v[0].x, 0x05040100u);
-                        o[0].y = __builtin_amdgcn_perm(v[3].x, v[2].x, 0x05040100u);
-                        o[1].x = __builtin_amdgcn_perm(v[1].x, v[0].x, 0x07060302u);
-                        o[1].y = __builtin_amdgcn_perm(v[3].x, v[2].x, 0x07060302u);
-                        o[2].x = __builtin_amdgcn_perm(v[1].y, v[0].y, 0x05040100u);
-                        o[2].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x05040100u);
-                        o[3].x = __builtin_amdgcn_perm(v[1].y, v[0].y, 0x07060302u);
-                        o[3].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x07060302u);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            *reinterpret_cast<u32x2 *>(lds + wr_off + (uint32_t)i * (64u * 128u)) = o[i];
-                    }
-                    __syncthreads();
-
-                    // ---- lookups ----
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        if (!ractive[r])
-                            continue;
-                        // row offsets (128 B per activation code) of the channels of this fill
-                        uint32_t ax = 0, ay = 0;
-                        if (KS == 1) {
-                            ax = ((a4[r] >> (8 * sub)) & 0xffu) << 7;
-                        } else if (KS == 2) {
-                            ax = ((a4[r] >> (16 * sub)) & 0xffu) << 7;
-                            ay = ((a4[r] >> (16 * sub + 8)) & 0xffu) << 7;
-                        } else {
-                            ax = __builtin_amdgcn_alignbit(a4[r], a4[r], rot_kk0);
-                            ay = __builtin_amdgcn_alignbit(ax, ax, rot_p0);
-                        }
-#pragma unroll
-                        for (int s = 0; s < 8; ++s) {
-                            uint32_t aoff;
-                            if (KS == 1)
-                                aoff = ax;
-                            else if (KS == 2)
-                                aoff = kk_hi[s] ? ay : ax;
-                            else
-                                aoff = ((((s & 1) ? ay : ax) >> (8 * (s >> 1))) & 0xffu) << 7;
-                            const u32x4 e = *reinterpret_cast<const u32x4 *>(lds + aoff + choff[s]);
-                            int32_t *a = &acc[r][(s & (SETS - 1)) * 8];
-                            a[0] += (int32_t)(e.x & 0xffffu);
-                            a[1] += (int32_t)(e.x >> 16);
-                            a[2] += (int32_t)(e.y & 0xffffu);
-                            a[3] += (int32_t)(e.y >> 16);
-                            a[4] += (int32_t)(e.z & 0xffffu);
-                            a[5] += (int32_t)(e.z >> 16);
-                            a[6] += (int32_t)(e.w & 0xffffu);
-                            a[7] += (int32_t)(e.w >> 16);
-                        }
-                    }
-                }
             }
+            if (fill + 2 < fills)
+                wn = *reinterpret_cast<const u32x2 *>(wq_tile + (size_t)(fill + 2) * 64);
         }
 
         // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----

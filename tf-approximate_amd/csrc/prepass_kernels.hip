@@ -39,6 +39,27 @@ __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__r
         chsum[pix] = sum;
 }
 
+// Same result as quantize_relayout_kernel for C % 4 == 0, with fully coalesced reads: consecutive lanes
+// read consecutive float4 of the NHWC input (one float4 = the four channels of one xq dword).
+__global__ void __launch_bounds__(256) quantize_relayout_vec4_kernel(const float4 *__restrict__ x4, int64_t quads,
+                                                                      int W, int C4, float offset, float inv_scale,
+                                                                      uint32_t *__restrict__ xq)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) {
+        const float4 v = x4[i];
+        const int64_t pix = i / C4;
+        const int c4 = (int)(i - pix * C4);
+        const int64_t nh = pix / W;
+        const int w = (int)(pix - nh * W);
+        const uint32_t packed = phys_row(quantize_code(v.x, offset, inv_scale)) |
+                                (phys_row(quantize_code(v.y, offset, inv_scale)) << 8) |
+                                (phys_row(quantize_code(v.z, offset, inv_scale)) << 16) |
+                                (phys_row(quantize_code(v.w, offset, inv_scale)) << 24);
+        xq[(nh * C4 + c4) * W + w] = packed;
+    }
+}
+
 // Patch sums (the outCoeffs of ApproxConvIm2ColKernel, tf2/src/approx_nn_conv_kernels.cpp:294): for each
 // output pixel the fp32 sum of the raw input over its patch, accumulated strictly in the reference's order
 // (kh, kw, c ascending; taps outside the image add 0.0f, which leaves the sum unchanged).  fp32 addition is
@@ -80,6 +101,66 @@ __global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict
         }
     }
     psum[m] = s;
+}
+
+// Patch sums for C % 4 == 0, same order and same results as patch_sums_kernel.  One thread per output
+// pixel still owns the sequential chain, but the floats arrive through LDS: for each tap the block loads
+// the 256 input pixels of its 256 output pixels cooperatively (8 lanes read the 128 contiguous bytes of a
+// 32-channel slice of one pixel), so a wavefront touches 8 memory lines per load instead of 64.
+constexpr int kPsTile = 256;  // output pixels per block
+constexpr int kPsCh = 32;     // channels per LDS slice
+constexpr int kPsRow = kPsCh + 4; // padded row (floats): conflict-free 16-byte accesses
+
+__global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *__restrict__ x, ConvGeom g,
+                                                                    float *__restrict__ psum)
+{
+    __shared__ int64_t bases[kPsTile];
+    __shared__ __align__(16) float tile[kPsTile * kPsRow];
+    const int t = threadIdx.x;
+    const int64_t m = (int64_t)blockIdx.x * kPsTile + t;
+    const bool valid = m < g.M;
+    int n = 0, ih0 = 0, iw0 = 0;
+    if (valid) {
+        n = (int)(m / ((int64_t)g.OH * g.OW));
+        const int rem = (int)(m - (int64_t)n * g.OH * g.OW);
+        const int oh = rem / g.OW, ow = rem - oh * g.OW;
+        ih0 = oh * g.sh - g.ph;
+        iw0 = ow * g.sw - g.pw;
+    }
+    float s = 0.0f;
+    constexpr int kQuads = kPsCh / 4;                       // float4 per pixel per slice
+    constexpr int kLoads = kPsTile * kQuads / kPsTile;      // float4 loads per thread per slice
+    for (int kh = 0; kh < g.KH; ++kh)
+        for (int kw = 0; kw < g.KW; ++kw) {
+            const int ih = ih0 + kh * g.dh, iw = iw0 + kw * g.dw;
+            const bool inb = valid && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+            __syncthreads(); // previous slice consumed
+            bases[t] = inb ? (((int64_t)n * g.H + ih) * g.W + iw) * g.C : (int64_t)-1;
+            for (int c0 = 0; c0 < g.C; c0 += kPsCh) {
+                __syncthreads(); // bases visible / previous slice consumed
+#pragma unroll
+                for (int i = 0; i < kLoads; ++i) {
+                    const int idx = t + i * kPsTile;
+                    const int pl = idx / kQuads, j = idx % kQuads;
+                    const int64_t b = bases[pl];
+                    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    if (b >= 0 && c0 + j * 4 < g.C)
+                        v = *reinterpret_cast<const float4 *>(x + b + c0 + j * 4);
+                    *reinterpret_cast<float4 *>(&tile[pl * kPsRow + j * 4]) = v;
+                }
+                __syncthreads();
+                const int nq = (g.C - c0 < kPsCh ? g.C - c0 : kPsCh) / 4;
+                for (int j = 0; j < nq; ++j) {
+                    const float4 v = *reinterpret_cast<const float4 *>(&tile[t * kPsRow + j * 4]);
+                    s = __fadd_rn(s, v.x);
+                    s = __fadd_rn(s, v.y);
+                    s = __fadd_rn(s, v.z);
+                    s = __fadd_rn(s, v.w);
+                }
+            }
+        }
+    if (valid)
+        psum[m] = s;
 }
 
 // Same relayout for caller-supplied codes (uint8 NHWC).
@@ -142,16 +223,36 @@ __global__ void __launch_bounds__(256) filter_pack_kernel(const float *__restric
 
 // Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one thread per output column,
 // rows (h, w, c) ascending.
+// A block owns 64 columns; all 256 threads stage 128 filter rows at a time into LDS (coalesced, many loads in
+// flight), then the first 64 threads extend their column's sequential sum from LDS.
 __global__ void __launch_bounds__(256) filter_sums_kernel(const float *__restrict__ filter, int K, int Co,
                                                            float *__restrict__ fsum)
 {
-    const int col = blockIdx.x * blockDim.x + threadIdx.x;
-    if (col >= Co)
-        return;
+    constexpr int kRows = 128;
+    __shared__ float stage[kRows * 65];
+    const int col0 = blockIdx.x * 64;
+    const int t = threadIdx.x;
+    const int cl = t & 63, rsub = t >> 6; // 4 rows per pass
     float s = 0.0f;
-    for (int k = 0; k < K; ++k)
-        s = __fadd_rn(s, filter[(int64_t)k * Co + col]);
-    fsum[col] = s;
+    for (int k0 = 0; k0 < K; k0 += kRows) {
+        __syncthreads();
+#pragma unroll 8
+        for (int r = rsub; r < kRows; r += 4) {
+            const int k = k0 + r;
+            float v = 0.0f;
+            if (k < K && col0 + cl < Co)
+                v = filter[(int64_t)k * Co + col0 + cl];
+            stage[r * 65 + cl] = v;
+        }
+        __syncthreads();
+        if (t < 64) {
+            const int nr = (K - k0 < kRows) ? K - k0 : kRows;
+            for (int r = 0; r < nr; ++r)
+                s = __fadd_rn(s, stage[r * 65 + t]);
+        }
+    }
+    if (t < 64 && col0 + t < Co)
+        fsum[col0 + t] = s;
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -186,6 +287,14 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float off
                                     uint32_t *xq, float *chsum, hipStream_t stream)
 {
     const int64_t pixels = (int64_t)g.N * g.H * g.W;
+    if ((g.C & 3) == 0 && !chsum && ((uintptr_t)x & 15) == 0) {
+        const int64_t quads = pixels * g.C4;
+        int64_t blocks = (quads + 256 * 4 - 1) / (256 * 4);
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(quantize_relayout_vec4_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           reinterpret_cast<const float4 *>(x), quads, g.W, g.C4, offset, inv_scale, xq);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(quantize_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, x, pixels,
                        g.H, g.W, g.C, g.C4, offset, inv_scale, xq, chsum);
     return hipGetLastError();
@@ -193,7 +302,11 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float off
 
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream)
 {
-    hipLaunchKernelGGL(patch_sums_kernel, dim3(blocks_for(g.M, 256)), dim3(256), 0, stream, x, g, psum);
+    if ((g.C & 3) == 0 && ((uintptr_t)x & 15) == 0)
+        hipLaunchKernelGGL(patch_sums_tiled_kernel, dim3(blocks_for(g.M, kPsTile)), dim3(kPsTile), 0, stream, x, g,
+                           psum);
+    else
+        hipLaunchKernelGGL(patch_sums_kernel, dim3(blocks_for(g.M, 256)), dim3(256), 0, stream, x, g, psum);
     return hipGetLastError();
 }
 
@@ -216,7 +329,7 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !fsum || !filter)
         return e;
-    hipLaunchKernelGGL(filter_sums_kernel, dim3(blocks_for(g.Co, 256)), dim3(256), 0, stream, filter, g.K, g.Co,
+    hipLaunchKernelGGL(filter_sums_kernel, dim3(blocks_for(g.Co, 64)), dim3(256), 0, stream, filter, g.K, g.Co,
                        fsum);
     return hipGetLastError();
 }
