@@ -13,7 +13,7 @@
 using namespace axc;
 
 struct axc_table {
-    uint16_t *dev_tableT; // [256 filter code][256 input code]
+    uint16_t *dev_tableT; // [257 filter code][256 input code]; row 256 is zero
     int device;
 };
 
@@ -244,6 +244,10 @@ int validate_for_launch(const axc_conv2d_desc *d, const axc_conv2d_dims &dm, boo
     const int64_t in_elems = (int64_t)dm.batch * dm.input_rows * dm.input_cols * dm.in_depth;
     if (out_elems >= ((int64_t)1 << 40) || in_elems >= ((int64_t)1 << 40))
         return fail(AXC_INVALID_ARGUMENT, "tensor too large");
+    // the dense kernel addresses the quantized input with 32-bit byte offsets
+    const int64_t xq_bytes = ((int64_t)dm.batch * dm.input_rows + 1) * dm.input_cols * ((dm.in_depth + 3) / 4) * 4;
+    if (!depthwise && xq_bytes >= ((int64_t)1 << 31))
+        return fail(AXC_INVALID_ARGUMENT, "input too large: more than 2^31 quantized activations");
     return AXC_OK;
 }
 
@@ -280,10 +284,10 @@ DensePlan make_plan(const ConvGeom &g, int cus)
     for (int nt : {16, 32, 64}) {
         if (nt > 16 && nt / 2 >= g.Co)
             continue; // half the columns of a wider tile would be padding
-        const int R = 64 / nt, ks = 64 / nt, subs = 4 / ks;
+        const int R = 2 * (64 / nt), ks = 64 / nt, subs = 4 / ks;
         const int n_col = (g.Co + nt - 1) / nt;
         const int fills = taps * g.C4 * subs;
-        const int64_t cap_wrows = (int64_t)kWaves * R; // wavefront-rows (64 pixels each) per tile
+        const int64_t cap_wrows = (int64_t)kDenseWaves * R; // wavefront-rows (64 pixels each) per tile
         const int64_t total_wrows = (g.M + 63) / 64;
         const int64_t min_tiles = (total_wrows + cap_wrows - 1) / cap_wrows;
         // candidate row-tile counts: the minimum, and counts that fill whole rounds of CUs
@@ -328,7 +332,7 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
 {
     DenseWorkspace w;
     size_t off = 0;
-    w.xq_off = off; off += align_up((size_t)g.N * g.H * g.C4 * g.W * 4);
+    w.xq_off = off; off += align_up(((size_t)g.N * g.H + 1) * g.C4 * g.W * 4); // + the zero-point row
     w.psum_off = off; off += align_up((size_t)g.M * 4); // patch sums: one float per output pixel
     w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
     w.fsum_off = off; off += align_up((size_t)g.Co * 4);
@@ -415,12 +419,13 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     uint16_t *wq = reinterpret_cast<uint16_t *>(ws + pd.ws.wq_off);
     float *fsum = reinterpret_cast<float *>(ws + pd.ws.fsum_off);
 
+    const uint32_t zp4 = phys_row((uint32_t)qp.input_zero_code) * 0x01010101u;
     if (codes_mode) {
         ProfScope ps("codes_relayout", stream);
-        AXC_HIP(launch_codes_relayout(input_codes, g, xq, stream));
+        AXC_HIP(launch_codes_relayout(input_codes, g, zp4, xq, stream));
     } else {
         ProfScope ps("quantize_relayout", stream);
-        AXC_HIP(launch_quantize_relayout(input, g, qp.input_offset, qp.input_inv_scale, xq, nullptr, stream));
+        AXC_HIP(launch_quantize_relayout(input, g, qp.input_offset, qp.input_inv_scale, zp4, xq, nullptr, stream));
     }
     if (out_f && !codes_mode) {
         ProfScope ps("patch_sums", stream);
@@ -449,8 +454,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         volatile float km = (float)g.K * qp.m1xm2;
         p.k_m1xm2 = km;
     }
-    const uint32_t zp = phys_row((uint32_t)qp.input_zero_code);
-    p.zp4 = zp * 0x01010101u;
+    p.zp4 = zp4;
+    p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
+    p.wq_bytes = (uint32_t)((size_t)pd.plan.n_col_tiles * pd.plan.fills * 128);
     {
         ProfScope ps("lutgemm_expand", stream);
         AXC_HIP(launch_dense(p, out_i != nullptr, stream));
@@ -544,7 +550,7 @@ int axc_table_create(const uint16_t *host_table, axc_table **out)
     if (!host_table || !out)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
     // transpose to weight-code major: tableT[b][a] = T[(a << 8) | b]
-    std::vector<uint16_t> t(65536);
+    std::vector<uint16_t> t((size_t)kTableRows * 256, 0); // row 256 stays zero: the null weight's row
     for (int a = 0; a < 256; ++a)
         for (int b = 0; b < 256; ++b)
             t[(size_t)b * 256 + a] = host_table[(size_t)a * 256 + b];
@@ -552,9 +558,9 @@ int axc_table_create(const uint16_t *host_table, axc_table **out)
     tab->dev_tableT = nullptr;
     hipError_t e = hipGetDevice(&tab->device);
     if (e == hipSuccess)
-        e = hipMalloc(reinterpret_cast<void **>(&tab->dev_tableT), kTableBytes);
+        e = hipMalloc(reinterpret_cast<void **>(&tab->dev_tableT), kTableAllocBytes);
     if (e == hipSuccess)
-        e = hipMemcpy(tab->dev_tableT, t.data(), kTableBytes, hipMemcpyHostToDevice);
+        e = hipMemcpy(tab->dev_tableT, t.data(), kTableAllocBytes, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
         if (tab->dev_tableT)
             (void)hipFree(tab->dev_tableT);

@@ -9,13 +9,17 @@
 
 namespace axc {
 
-// LDS budget of one workgroup (the whole CU: 160 KiB).
 constexpr int kTableBytes = 131072;            // 256 x 256 uint16, weight-code major
-constexpr int kExpandBytes = 32768;            // 256 activation rows x 64 slots x uint16
-constexpr int kLdsBytes = kTableBytes + kExpandBytes;
-constexpr int kBlockThreads = 1024;            // 16 wavefronts: one workgroup per CU
+constexpr int kTableRows = 257;                // row 256 is all zeros: the row of the null weight
+constexpr int kTableAllocBytes = kTableRows * 512;
+constexpr int kExpandBytes = 32768;            // one expanded-row buffer: 256 activation rows x 64 slots x uint16
+constexpr int kDenseLdsBytes = 4 * kExpandBytes; // dense kernel: 2 buffers of expanded rows + 2 of staged table rows
+constexpr int kDenseThreads = 512;             // dense kernel: 8 wavefronts x 256 VGPRs, one workgroup per CU
+constexpr int kDenseWaves = kDenseThreads / 64;
+constexpr int kDenseParkBytes = 16 * 4 * kDenseThreads; // per-thread pixel geometry parked behind the buffers
+constexpr int kBlockThreads = 1024;            // depthwise kernel / LDS probe: 16 wavefronts per CU
 constexpr int kWaves = kBlockThreads / 64;
-constexpr uint16_t kNullWeight = 0xFFFF;       // slot that contributes nothing (padding channel / column)
+constexpr uint16_t kNullWeight = 256;          // slot that contributes nothing (padding channel / column)
 
 // Geometry of one dense layer after validation.
 struct ConvGeom {
@@ -40,15 +44,17 @@ struct DensePlan {
 struct DenseParams {
     ConvGeom g;
     DensePlan plan;
-    const uint32_t *xq;     // [N][H][C4][W] dwords of 4 row-permuted activation codes
+    const uint32_t *xq;     // [N][H][C4][W] dwords of 4 row-permuted activation codes, then one more
+                            // [C4][W] row holding the zero-point code (read by taps outside the image)
     const float *psum;      // [M] sum of the raw input over each output pixel's patch (float epilogue only)
     const uint16_t *wq;     // [n_col_tiles][fills][64] packed filter codes (kNullWeight = none)
     const float *fsum;      // [Co] sum over (h, w, c) of the raw filter
-    const uint16_t *tableT; // [256 filter code][256 input code]
+    const uint16_t *tableT; // [257 filter code (256 = null)][256 input code]
     float *out_f;
     int32_t *out_i;
     float s1xs2, m1, m2, k_m1xm2; // epilogue constants; k_m1xm2 = float(K) * m1xM2
     uint32_t zp4;           // row-permuted zero code replicated in all four bytes
+    uint32_t xq_bytes, wq_bytes; // sizes of the two streams (buffer-descriptor bounds)
 };
 
 struct DepthwiseParams {
@@ -80,9 +86,10 @@ __device__ inline uint32_t quantize_code(float v, float offset, float inv_scale)
 
 // ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
 hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
-                                    uint32_t *xq, float *chsum, hipStream_t stream);
+                                    uint32_t zp4, uint32_t *xq, float *chsum, hipStream_t stream);
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream);
-hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t *xq, hipStream_t stream);
+hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
+                                 hipStream_t stream);
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
                               const DensePlan &plan, float offset, float inv_scale,
                               uint16_t *wq, float *fsum, hipStream_t stream);

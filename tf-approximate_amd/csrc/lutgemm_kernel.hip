@@ -1,21 +1,30 @@
 // Dense LUT-GEMM for gfx950: implicit-GEMM gather + table lookups out of LDS + fused epilogue.
 //
-// One workgroup (16 wavefronts) owns a CU and its 160 KiB of LDS:
-//   [0, 128 KiB)        the whole truth table, weight-code major: row b holds T[a][b] for a = 0..255
-//   [128 KiB, 160 KiB)  the "expanded rows": for the 64 weight slots of the current fill,
-//                       E[phys_row(a)][slot] = T[a][code(slot)], 128 bytes per activation code
+// A "fill" takes 64 filter entries (KS consecutive input channels x NT output columns, KS * NT = 64) and
+// builds their expanded rows in LDS: E[phys_row(a)][slot] = T[a][code(slot)], 128 bytes per activation
+// code a, 32 KiB per fill.  Every lane then looks up, for each of its R output pixels, the expanded row of
+// its activation code with ds_read_b128: eight table entries per LDS access instead of one, and the
+// 16-byte chunks the lanes of a wavefront touch in one instruction are rotated by lane so they fall into
+// different banks whatever the activation codes are.  Sums are exact int32.
 //
-// A fill takes 64 filter entries (KS consecutive input channels x NT output columns, KS * NT = 64),
-// copies the table row of each entry into the expanded area transposed (derive phase), then every
-// lane looks up, for each of its R = 64 / NT output pixels, the expanded row of its activation code
-// with ds_read_b128: eight table entries per LDS access instead of one, and the 16-byte chunks the
-// lanes of a wavefront touch in one instruction are rotated by lane so they fall into different
-// banks whatever the activation codes are.  Sums are exact int32.
+// Everything is double-buffered in LDS so that one barrier per fill is all the synchronization there is:
+//   expanded rows   2 x 32 KiB  wavefronts look up fill p out of one buffer while they transpose the
+//                               table rows of fill p + 1 into the other
+//   staged rows     2 x 32 KiB  the 64 table rows (512 contiguous bytes per filter code) of fill p + 1,
+//                               read bank-conflict free by the transposing lanes, while the rows of fill
+//                               p + 2 land in the other buffer
+// The table itself (128 KiB, resident in L2) is read with fully coalesced 16-byte loads, half a wavefront per
+// row, three fills ahead of the lookups; the filter codes that select the rows four fills ahead.
+//
+// One workgroup of 8 wavefronts per CU, 256 VGPRs per wavefront: 128 int32 accumulators per lane
+// (R = 8 pixels x 16 columns, 4 x 32 or 2 x 64), eight 16-byte lookups in flight per wavefront.
 //
 // Restates, as one fused kernel, what the reference does in ApproxConvIm2ColKernel +
 // ApproxConvGEMMKernel (tf2/src/approx_nn_conv_kernels.cpp:215-296) per chunk.
 #include "axconv_internal.h"
 #include "lookup_asm.inc"
+
+#include <type_traits>
 
 namespace axc {
 
@@ -24,68 +33,113 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 extern __shared__ __align__(16) unsigned char lds[];
 
-// Four table-row reads in flight, then one wait: the compiler would serialize them.
-__device__ __forceinline__ void lds_read4_b64(uint64_t (&v)[4], const uint32_t (&addr)[4])
+// Global loads go through raw buffer descriptors: address = SGPR base + SGPR offset + one 32-bit VGPR
+// offset, so no load needs a 64-bit VGPR address, and reads past the end return 0 instead of faulting.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes)
 {
-    asm volatile("ds_read_b64 %0, %4\n\t"
-                 "ds_read_b64 %1, %5\n\t"
-                 "ds_read_b64 %2, %6\n\t"
-                 "ds_read_b64 %3, %7\n\t"
-                 "s_waitcnt lgkmcnt(0)"
-                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
-                 : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3])
-                 : "memory");
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint32_t ld_u32(rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
+}
+__device__ __forceinline__ u32x2 ld_u32x2(rsrc_t r, uint32_t voff, uint32_t soff)
+{
+    return __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0);
+}
+
+template <int NT>
+struct DenseCfg {
+    static constexpr int R = 2 * (64 / NT);   // output pixels per lane
+    static constexpr int KS = 64 / NT;        // input channels per fill
+    static constexpr int SETS = NT / 8;       // 8-column groups per pixel
+    static constexpr int SUBS = 4 / KS;       // fills per channel quad
+};
+
+// Lookups of one fill for the R output pixels of this lane (out of expanded-row buffer BUF).
+template <int NT, int BUF>
+__device__ __forceinline__ void lookup_rows(int32_t (&acc)[DenseCfg<NT>::R][NT], const uint32_t (&a4)[DenseCfg<NT>::R],
+                                            const int sub, const bool (&ractive)[DenseCfg<NT>::R],
+                                            const uint32_t (&choff)[8], const uint32_t rot_kk0, const uint32_t rot_p0,
+                                            const uint64_t (&kk_mask)[8])
+{
+    constexpr int R = DenseCfg<NT>::R, KS = DenseCfg<NT>::KS;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!ractive[r])
+            continue;
+        if constexpr (KS == 4) {
+            // rotate so that the channel of step s is byte s >> 1 of ax (even s) / ay (odd s)
+            const uint32_t ax = __builtin_amdgcn_alignbit(a4[r], a4[r], rot_kk0);
+            const uint32_t ay = __builtin_amdgcn_alignbit(ax, ax, rot_p0);
+            if constexpr (BUF == 0) LOOKUP_ROW_NT16_B0(acc[r], ax, ay, choff); else LOOKUP_ROW_NT16_B1(acc[r], ax, ay, choff);
+        } else if constexpr (KS == 2) {
+            const uint32_t ax = ((a4[r] >> (16 * sub)) & 0xffu) << 7;      // row offsets of the two channels
+            const uint32_t ay = ((a4[r] >> (16 * sub + 8)) & 0xffu) << 7;
+            if constexpr (BUF == 0) LOOKUP_ROW_NT32_B0(acc[r], ax, ay, choff, kk_mask); else LOOKUP_ROW_NT32_B1(acc[r], ax, ay, choff, kk_mask);
+        } else {
+            const uint32_t ax = ((a4[r] >> (8 * sub)) & 0xffu) << 7;
+            if constexpr (BUF == 0) LOOKUP_ROW_NT64_B0(acc[r], ax, ax, choff); else LOOKUP_ROW_NT64_B1(acc[r], ax, ax, choff);
+        }
+    }
 }
 
 template <int NT, bool OUT_I32>
-__global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const DenseParams p)
+__global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const DenseParams p)
 {
-    constexpr int R = 64 / NT;        // output pixels per lane
-    constexpr int KS = 64 / NT;       // input channels per fill
-    constexpr int SETS = NT / 8;      // 8-column groups per pixel
-    constexpr int SUBS = 4 / KS;      // fills per channel quad
+    constexpr int R = DenseCfg<NT>::R, SETS = DenseCfg<NT>::SETS, SUBS = DenseCfg<NT>::SUBS;
     constexpr int LOG_SETS = (SETS == 8) ? 3 : (SETS == 4) ? 2 : 1;
+    constexpr int ITEMS = 16 / kDenseWaves; // derive items (4 activation codes x 4 slots) per thread per fill
 
     const ConvGeom &g = p.g;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: row activity branches on SGPRs
 
-    // ---- stage the truth table (once per workgroup; the workgroup is persistent) ----
-    {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(p.tableT);
-        u32x4 *dst = reinterpret_cast<u32x4 *>(lds);
-#pragma unroll
-        for (int i = 0; i < kTableBytes / 16 / kBlockThreads; ++i)
-            dst[tid + i * kBlockThreads] = src[tid + i * kBlockThreads];
-    }
-
     // ---- lane constants ----
     const int c0 = lane & 7;
-    uint32_t choff[8];   // byte offset of the chunk this lane reads at step s
+    uint32_t choff[8];   // byte offset, inside an expanded row, of the chunk this lane reads at step s
 #pragma unroll
     for (int s = 0; s < 8; ++s)
-        choff[s] = (uint32_t)kTableBytes + ((uint32_t)((c0 + s) & 7) << 4);
+        choff[s] = (uint32_t)((c0 + s) & 7) << 4;
     // The chunk of step s belongs to input channel kk_s = ((c0 + s) & 7) >> LOG_SETS of the fill.
     // KS == 4: kk_s = (kk0 + ((p0 + s) >> 1)) & 3 with kk0 = c0 >> 1, p0 = c0 & 1, so after rotating the
     //          activation dword right by kk0 bytes (and by p0 more for odd s) the byte index is the
     //          compile-time constant s >> 1.
-    // KS == 2: kk_s is one bit; it is kept as a per-step lane mask.
+    // KS == 2: kk_s is one bit, kept as a per-step lane mask in SGPRs.
     const uint32_t rot_kk0 = (uint32_t)(c0 >> 1) << 3;
     const uint32_t rot_p0 = (uint32_t)(c0 & 1) << 3;
-    bool kk_hi[8];
+    uint64_t kk_mask[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s)
-        kk_hi[s] = ((((c0 + s) & 7) >> LOG_SETS) & 1) != 0;
-    // derive phase: lane transposes activation codes 4*lane .. 4*lane+3 for slots 4*jq .. 4*jq+3
-    const int jq = (lane + wave) & 15;
-    const uint32_t rd_off = (uint32_t)lane * 8u;
-    const uint32_t wr_off = (uint32_t)kTableBytes + (uint32_t)lane * 128u + (uint32_t)jq * 8u;
+        kk_mask[s] = __ballot(((((c0 + s) & 7) >> LOG_SETS) & 1) != 0);
+    // derive: item i of this lane transposes activation codes 4*lane .. 4*lane+3 of the staged table rows of
+    // slots 4*jq_i .. 4*jq_i+3; the row permutation phys_row() and the rotation of jq by wavefront make
+    // both the staged-row reads and the expanded-row writes bank-conflict free
+    uint32_t jq8[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i)
+        jq8[i] = (uint32_t)((lane + wave + i * kDenseWaves) & 15) * 8u; // byte offset of 4 slots in a row
+    const uint32_t rd_lane = (uint32_t)lane * 8u;    // this lane's 8 bytes inside a staged 512-byte row
+    const uint32_t wr_row = (uint32_t)lane * 128u;
+    // staging: load j of this thread fetches 16 bytes of the table row of slot 16*j + tid/32
+    const uint32_t st_slot = (uint32_t)tid >> 5;
+    const uint32_t st_off = ((uint32_t)tid & 31u) * 16u;
+    // per-thread geometry is parked in LDS behind the four buffers: [slot][thread]
+    uint32_t *const park = reinterpret_cast<uint32_t *>(lds + kDenseLdsBytes) + tid;
+    unsigned char *const stage = lds + 2 * kExpandBytes;
 
     const int taps = g.KH * g.KW;
     const int ntiles = p.plan.n_row_tiles * p.plan.n_col_tiles;
     const int fills = p.plan.fills;
     const int rowstep = g.C4 * g.W; // dwords between input rows in xq
+    // xq ends with one extra input row filled with the zero-point code: taps outside the image read it
+    const uint32_t zp_row = p.xq_bytes;
+    const rsrc_t xq_rsrc = make_rsrc(p.xq, p.xq_bytes + (uint32_t)rowstep * 4u);
+    const rsrc_t wq_rsrc = make_rsrc(p.wq, p.wq_bytes);
+    const rsrc_t tab_rsrc = make_rsrc(p.tableT, (uint32_t)kTableAllocBytes);
+    (void)taps;
 
     for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int ct = tile % p.plan.n_col_tiles;
@@ -93,14 +147,12 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
         const int64_t row0 = (int64_t)rt * p.plan.rows_per_tile;
         const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
 
-        // ---- per-pixel geometry ----
-        int32_t pbase[R];  // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
-        int hw0[R];        // (ih0 << 16) | (iw0 & 0xffff): input coordinates of tap (0, 0)
+        // ---- per-pixel geometry (parked in LDS; only read back when the tap changes) ----
         bool rvalid[R];    // this lane's pixel exists
         bool ractive[R];   // some lane of this wavefront has a pixel (wave-uniform)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int64_t wrow = row0 + (int64_t)(r * kWaves + wave) * 64;
+            const int64_t wrow = row0 + (int64_t)(r * kDenseWaves + wave) * 64;
             ractive[r] = wrow < row_end;
             const int64_t m = wrow + lane;
             rvalid[r] = m < row_end;
@@ -110,8 +162,10 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
             const int oh = rem / g.OW;
             const int ow = rem - oh * g.OW;
             const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
-            pbase[r] = (n * g.H + ih0) * rowstep + iw0;
-            hw0[r] = (ih0 << 16) | (iw0 & 0xffff);
+            // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
+            park[(2 * r) * kDenseThreads] = (uint32_t)((n * g.H + ih0) * rowstep + iw0);
+            // input coordinates of tap (0, 0); ih0 = -32768 marks a pixel that does not exist
+            park[(2 * r + 1) * kDenseThreads] = rvalid[r] ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
         }
 
         int32_t acc[R][NT];
@@ -121,154 +175,132 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
             for (int j = 0; j < NT; ++j)
                 acc[r][j] = 0;
 
-        const uint16_t *wq_tile = p.wq + (size_t)ct * fills * 64 + jq * 4;
+        const uint32_t wq_tile = (uint32_t)ct * (uint32_t)fills * 128u; // byte offset of this tile's codes
 
-        // ---- load cursor: (tap, quad) of the activation dwords to fetch next ----
-        int tap_n = 0, q_n = 0, kh_n = 0, kw_n = 0;
-        bool inb_n[R];
-        int32_t idx_n[R];
+        // ---- activation cursor: position (tap, quad) of the fill whose activations are fetched next ----
+        int cur_fill = 0, cur_q = 0, cur_kh = 0, cur_kw = 0, cur_sub = 0;
+        uint32_t idx_tap[R];   // byte offset in xq of quad 0 of the current tap (the zero-point row outside)
         auto tap_setup = [&]() {
-            const int dh = kh_n * g.dh, dw = kw_n * g.dw;
+            const int dh = cur_kh * g.dh, dw = cur_kw * g.dw;
+            const int tap_off = dh * rowstep + dw;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int ih = (hw0[r] >> 16) + dh;
-                const int iw = (int)(int16_t)(hw0[r] & 0xffff) + dw;
-                inb_n[r] = rvalid[r] && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-                idx_n[r] = inb_n[r] ? pbase[r] + dh * rowstep + dw : 0;
+                const int32_t pb = (int32_t)park[(2 * r) * kDenseThreads];
+                const int32_t hw = (int32_t)park[(2 * r + 1) * kDenseThreads];
+                const int ih = (hw >> 16) + dh;
+                const int iw = (int)(int16_t)(hw & 0xffff) + dw;
+                const bool inb = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+                idx_tap[r] = inb ? (uint32_t)((pb + tap_off) * 4) : zp_row;
             }
         };
-        uint32_t a4n[R];
-        auto issue_act_loads = [&]() {
-            // unconditional loads (index 0 when outside the image) keep the number of outstanding
-            // loads static, so waits on older loads do not have to drain these
+        auto load_acts = [&](uint32_t (&dst)[R]) {
+            const uint32_t qoff = (uint32_t)(cur_q * g.W * 4); // scalar: channel quad inside the pixel row
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const uint32_t v = p.xq[idx_n[r] + (inb_n[r] ? q_n * g.W : 0)];
-                a4n[r] = inb_n[r] ? v : p.zp4;
-            }
+            for (int r = 0; r < R; ++r)
+                dst[r] = ld_u32(xq_rsrc, idx_tap[r], qoff);
         };
-        auto advance_cursor = [&]() {
-            if (++q_n == g.C4) {
-                q_n = 0;
-                ++tap_n;
-                if (++kw_n == g.KW) { kw_n = 0; ++kh_n; }
-                if (tap_n < taps)
-                    tap_setup();
+        auto advance_cursor = [&]() { // to the next fill
+            ++cur_fill;
+            if (++cur_sub == SUBS) {
+                cur_sub = 0;
+                if (++cur_q == g.C4) {
+                    cur_q = 0;
+                    if (++cur_kw == g.KW) { cur_kw = 0; ++cur_kh; }
+                    if (cur_fill < fills)
+                        tap_setup();
+                }
             }
         };
 
-        // derive phase, split so the table-row reads can run before the barrier that frees the
-        // expanded area and only the four writes sit between the two barriers
-        u32x2 o[4];
-        auto derive_read = [&](const u32x2 wc) {
-            const uint32_t code[4] = {wc.x & 0xffffu, wc.x >> 16, wc.y & 0xffffu, wc.y >> 16};
-            uint32_t addr[4];
-            bool none[4];
+        // ---- table rows of one fill: global -> registers -> staged rows -> expanded rows ----
+        auto load_codes = [&](int fill, uint32_t (&codes)[4]) {
+            const uint32_t f = (uint32_t)(fill < fills ? fill : fills - 1);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                none[i] = code[i] == kNullWeight;
-                addr[i] = (none[i] ? 0u : code[i]) * 512u + rd_off;
-            }
-            uint64_t v[4];
-            lds_read4_b64(v, addr);
-            uint32_t x[4], y[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                x[i] = none[i] ? 0u : (uint32_t)v[i];
-                y[i] = none[i] ? 0u : (uint32_t)(v[i] >> 32);
-            }
-            o[0].x = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
-            o[0].y = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
-            o[1].x = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
-            o[1].y = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
-            o[2].x = __builtin_amdgcn_perm(y[1], y[0], 0x05040100u);
-            o[2].y = __builtin_amdgcn_perm(y[3], y[2], 0x05040100u);
-            o[3].x = __builtin_amdgcn_perm(y[1], y[0], 0x07060302u);
-            o[3].y = __builtin_amdgcn_perm(y[3], y[2], 0x07060302u);
+            for (int j = 0; j < 4; ++j)
+                codes[j] = __builtin_amdgcn_raw_buffer_load_b16(wq_rsrc, (int)((st_slot + 16u * j) * 2u),
+                                                                (int)(wq_tile + f * 128u), 0);
         };
-        auto derive_write = [&]() {
+        auto load_rows = [&](const uint32_t (&codes)[4], u32x4 (&rows)[4]) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<u32x2 *>(lds + wr_off + (uint32_t)i * (64u * 128u)) = o[i];
+            for (int j = 0; j < 4; ++j)
+                rows[j] = __builtin_amdgcn_raw_buffer_load_b128(tab_rsrc, (int)((codes[j] & 0xffffu) * 512u + st_off), 0, 0);
+        };
+        auto store_stage = [&](const u32x4 (&rows)[4], const uint32_t buf) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<u32x4 *>(stage + buf * kExpandBytes + (st_slot + 16u * j) * 512u + st_off) = rows[j];
+        };
+        auto derive = [&](const uint32_t buf) { // staged rows [buf] -> expanded rows [buf]
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                u32x2 v[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) // slot 4*jq + k = byte offset jq8/2 + k in units of rows
+                    v[k] = *reinterpret_cast<const u32x2 *>(stage + buf * kExpandBytes + (jq8[i] / 2u + k) * 512u + rd_lane);
+                u32x2 o[4];
+                o[0].x = __builtin_amdgcn_perm(v[1].x, v[0].x, 0x05040100u);
+                o[0].y = __builtin_amdgcn_perm(v[3].x, v[2].x, 0x05040100u);
+                o[1].x = __builtin_amdgcn_perm(v[1].x, v[0].x, 0x07060302u);
+                o[1].y = __builtin_amdgcn_perm(v[3].x, v[2].x, 0x07060302u);
+                o[2].x = __builtin_amdgcn_perm(v[1].y, v[0].y, 0x05040100u);
+                o[2].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x05040100u);
+                o[3].x = __builtin_amdgcn_perm(v[1].y, v[0].y, 0x07060302u);
+                o[3].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x07060302u);
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    *reinterpret_cast<u32x2 *>(lds + buf * kExpandBytes + wr_row + jq8[i] + (uint32_t)k * (64u * 128u)) = o[k];
+            }
         };
 
-        // ---- prologue: activations of quad 0, weights of fill 0 -> expanded rows of fill 0 ----
-        uint32_t a4[R];
+        // ---- prologue ----
+        // state entering phase p: expanded rows of fill p in D[p & 1]; staged rows of fill p+1 in S[(p+1) & 1];
+        // rows = table rows of fill p+2 (in flight); codes = filter codes of fill p+3 (in flight);
+        // acts[p & 1] = activations of fill p
+        uint32_t actA[R], actB[R];
+        u32x4 rows[4];
+        uint32_t codes[4];
         tap_setup();
-        issue_act_loads();
-        u32x2 wn = *reinterpret_cast<const u32x2 *>(wq_tile);
-        __syncthreads(); // table staged / previous tile's lookups done
-        derive_read(wn);
-        derive_write();
+        load_acts(actA);
+        load_codes(0, codes);
+        load_rows(codes, rows);       // fill 0
+        load_codes(1, codes);
+        __syncthreads();              // the previous tile's last phase is done with every buffer
+        store_stage(rows, 0);
+        load_rows(codes, rows);       // fill 1
+        load_codes(2, codes);
         __syncthreads();
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-            a4[r] = a4n[r];
-        advance_cursor();
-        if (tap_n < taps)
-            issue_act_loads();
-        if (fills > 1)
-            wn = *reinterpret_cast<const u32x2 *>(wq_tile + 64);
+        derive(0);
+        store_stage(rows, 1);
+        load_rows(codes, rows);       // fill 2
+        load_codes(3, codes);
+        __syncthreads();
 
-        int sub = 0;
-        for (int fill = 0; fill < fills; ++fill) {
-            // ---- lookups of this fill ----
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (!ractive[r])
-                    continue;
-                // row offsets (128 B per activation code) of the channels of this fill
-                uint32_t ax = 0, ay = 0;
-                if (KS == 1) {
-                    ax = ((a4[r] >> (8 * sub)) & 0xffu) << 7;
-                } else if (KS == 2) {
-                    ax = ((a4[r] >> (16 * sub)) & 0xffu) << 7;
-                    ay = ((a4[r] >> (16 * sub + 8)) & 0xffu) << 7;
-                } else {
-                    ax = __builtin_amdgcn_alignbit(a4[r], a4[r], rot_kk0);
-                    ay = __builtin_amdgcn_alignbit(ax, ax, rot_p0);
-                }
-                uint32_t ad[8];
-#pragma unroll
-                for (int s = 0; s < 8; ++s) {
-                    uint32_t aoff;
-                    if (KS == 1)
-                        aoff = ax;
-                    else if (KS == 2)
-                        aoff = kk_hi[s] ? ay : ax;
-                    else
-                        aoff = ((((s & 1) ? ay : ax) >> (8 * (s >> 1))) & 0xffu) << 7;
-                    ad[s] = aoff + choff[s];
-                }
-                if constexpr (NT == 16) {
-                    LOOKUP_ROW_NT16(acc[r], ad);
-                } else if constexpr (NT == 32) {
-                    LOOKUP_ROW_NT32(acc[r], ad);
-                } else {
-                    LOOKUP_ROW_NT64(acc[r], ad);
-                }
+        // One phase: expand the next fill, stage the one after, issue the loads behind them, look up.
+        auto phase = [&](const int pcur, uint32_t (&act_cur)[R], uint32_t (&act_next)[R], auto buf_tag) {
+            constexpr int BUF = decltype(buf_tag)::value;
+            const int sub = cur_sub; // sub-step of fill pcur inside its channel quad
+            // 1. consume what earlier phases loaded (nothing here waits on a fresh load)
+            if (pcur + 1 < fills)
+                derive(BUF ^ 1);          // fill pcur+1: staged rows -> expanded rows
+            if (pcur + 2 < fills)
+                store_stage(rows, BUF);   // fill pcur+2: registers -> staged rows (derive(pcur) read this buffer a phase ago)
+            __builtin_amdgcn_sched_barrier(0);
+            // 2. issue the loads later phases consume
+            if (pcur + 1 < fills) {
+                load_rows(codes, rows);       // fill pcur+3
+                load_codes(pcur + 4, codes);
+                advance_cursor();             // cursor -> fill pcur+1
+                load_acts(act_next);
             }
-            if (fill + 1 == fills)
-                break;
-
-            // ---- expanded rows of the next fill ----
-            derive_read(wn);   // table-row reads + transposes overlap other wavefronts' lookups
-            __syncthreads();   // every wavefront is done reading the expanded rows of this fill
-            derive_write();
+            __builtin_amdgcn_sched_barrier(0);
+            // 3. look up
+            lookup_rows<NT, BUF>(acc, act_cur, sub, ractive, choff, rot_kk0, rot_p0, kk_mask);
             __syncthreads();
-
-            // ---- roll the pipeline: consume the prefetched registers, then issue the next loads ----
-            if (++sub == SUBS) {
-                sub = 0;
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    a4[r] = a4n[r];
-                advance_cursor();
-                if (tap_n < taps)
-                    issue_act_loads();
-            }
-            if (fill + 2 < fills)
-                wn = *reinterpret_cast<const u32x2 *>(wq_tile + (size_t)(fill + 2) * 64);
+        };
+        for (int pcur = 0; pcur < fills; pcur += 2) {
+            phase(pcur, actA, actB, std::integral_constant<int, 0>());
+            if (pcur + 1 < fills)
+                phase(pcur + 1, actB, actA, std::integral_constant<int, 1>());
         }
 
         // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----
@@ -276,7 +308,7 @@ __global__ void __launch_bounds__(kBlockThreads) lutgemm_expand_kernel(const Den
         for (int r = 0; r < R; ++r) {
             if (!rvalid[r])
                 continue;
-            const int64_t m = row0 + (int64_t)(r * kWaves + wave) * 64 + lane;
+            const int64_t m = row0 + (int64_t)(r * kDenseWaves + wave) * 64 + lane;
             // patch sum of the raw input in the reference's order (tap-major, channels ascending)
             const float psum = OUT_I32 ? 0.0f : p.psum[m];
             const float t1 = __fmul_rn(p.m2, psum);
@@ -310,10 +342,10 @@ static hipError_t launch_one(const DenseParams &p, hipStream_t stream)
 {
     auto kernel = lutgemm_expand_kernel<NT, OUT_I32>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDenseLdsBytes + kDenseParkBytes);
     if (e != hipSuccess)
         return e;
-    hipLaunchKernelGGL(kernel, dim3(p.plan.grid), dim3(kBlockThreads), kLdsBytes, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(p.plan.grid), dim3(kDenseThreads), kDenseLdsBytes + kDenseParkBytes, stream, p);
     return hipGetLastError();
 }
 

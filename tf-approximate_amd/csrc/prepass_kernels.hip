@@ -283,9 +283,28 @@ __global__ void __launch_bounds__(256) depthwise_filter_kernel(const float *__re
 
 static inline unsigned blocks_for(int64_t n, int threads) { return (unsigned)((n + threads - 1) / threads); }
 
-hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
-                                    uint32_t *xq, float *chsum, hipStream_t stream)
+// The extra [C4][W] row behind xq: every dword is the zero-point code x4.
+__global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t *__restrict__ dst, int n, uint32_t value)
 {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        dst[i] = value;
+}
+
+static hipError_t launch_zero_point_row(const ConvGeom &g, uint32_t zp4, uint32_t *xq, hipStream_t stream)
+{
+    const int n = g.C4 * g.W;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, stream,
+                       xq + (size_t)g.N * g.H * g.C4 * g.W, n, zp4);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
+                                    uint32_t zp4, uint32_t *xq, float *chsum, hipStream_t stream)
+{
+    hipError_t ez = launch_zero_point_row(g, zp4, xq, stream);
+    if (ez != hipSuccess)
+        return ez;
     const int64_t pixels = (int64_t)g.N * g.H * g.W;
     if ((g.C & 3) == 0 && !chsum && ((uintptr_t)x & 15) == 0) {
         const int64_t quads = pixels * g.C4;
@@ -310,8 +329,12 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hip
     return hipGetLastError();
 }
 
-hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t *xq, hipStream_t stream)
+hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
+                                 hipStream_t stream)
 {
+    hipError_t ez = launch_zero_point_row(g, zp4, xq, stream);
+    if (ez != hipSuccess)
+        return ez;
     const int64_t pixels = (int64_t)g.N * g.H * g.W;
     hipLaunchKernelGGL(codes_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, codes, pixels,
                        g.W, g.C, g.C4, xq);
