@@ -16,7 +16,16 @@ FLAGS = [
 ]
 
 
+def generate():
+    """Writes csrc/lookup_asm.inc, the generated inline assembly of the lookup phase."""
+    gen = os.path.join(CSRC, "gen_lookup_asm.py")
+    text = subprocess.run([sys.executable, gen], stdout=subprocess.PIPE, text=True, check=True).stdout
+    with open(os.path.join(CSRC, "lookup_asm.inc"), "w") as f:
+        f.write(text)
+
+
 def build(verbose=False, extra=()):
+    generate()
     cmd = ["hipcc"] + FLAGS + list(extra) + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
     if verbose:
         print(" ".join(cmd))

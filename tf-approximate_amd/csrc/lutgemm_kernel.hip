@@ -49,6 +49,8 @@ __device__ __forceinline__ u32x2 ld_u32x2(rsrc_t r, uint32_t voff, uint32_t soff
     return __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0);
 }
 
+constexpr int kOldShare = 11; // sixteenths of a tile's wavefront-rows owned by the older four wavefronts
+
 template <int NT>
 struct DenseCfg {
     static constexpr int R = 2 * (64 / NT);   // output pixels per lane
@@ -57,31 +59,18 @@ struct DenseCfg {
     static constexpr int SUBS = 4 / KS;       // fills per channel quad
 };
 
-// Lookups of one fill for the R output pixels of this lane (out of expanded-row buffer BUF).
+// Lookups of one fill for the first nr output pixels of this lane (out of expanded-row buffer BUF).
 template <int NT, int BUF>
-__device__ __forceinline__ void lookup_rows(int32_t (&acc)[DenseCfg<NT>::R][NT], const uint32_t (&a4)[DenseCfg<NT>::R],
-                                            const int sub, const bool (&ractive)[DenseCfg<NT>::R],
-                                            const uint32_t (&choff)[8], const uint32_t rot_kk0, const uint32_t rot_p0,
-                                            const uint64_t (&kk_mask)[8])
+__device__ __forceinline__ void lookup_fill(int32_t (&acc)[DenseCfg<NT>::R][NT], const uint32_t (&a4)[DenseCfg<NT>::R],
+                                            const uint32_t (&sel)[8], const uint32_t cha, const uint32_t chb,
+                                            const uint32_t nr, const uint32_t shift)
 {
-    constexpr int R = DenseCfg<NT>::R, KS = DenseCfg<NT>::KS;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        if (!ractive[r])
-            continue;
-        if constexpr (KS == 4) {
-            // rotate so that the channel of step s is byte s >> 1 of ax (even s) / ay (odd s)
-            const uint32_t ax = __builtin_amdgcn_alignbit(a4[r], a4[r], rot_kk0);
-            const uint32_t ay = __builtin_amdgcn_alignbit(ax, ax, rot_p0);
-            if constexpr (BUF == 0) LOOKUP_ROW_NT16_B0(acc[r], ax, ay, choff); else LOOKUP_ROW_NT16_B1(acc[r], ax, ay, choff);
-        } else if constexpr (KS == 2) {
-            const uint32_t ax = ((a4[r] >> (16 * sub)) & 0xffu) << 7;      // row offsets of the two channels
-            const uint32_t ay = ((a4[r] >> (16 * sub + 8)) & 0xffu) << 7;
-            if constexpr (BUF == 0) LOOKUP_ROW_NT32_B0(acc[r], ax, ay, choff, kk_mask); else LOOKUP_ROW_NT32_B1(acc[r], ax, ay, choff, kk_mask);
-        } else {
-            const uint32_t ax = ((a4[r] >> (8 * sub)) & 0xffu) << 7;
-            if constexpr (BUF == 0) LOOKUP_ROW_NT64_B0(acc[r], ax, ax, choff); else LOOKUP_ROW_NT64_B1(acc[r], ax, ax, choff);
-        }
+    if constexpr (NT == 16) {
+        if constexpr (BUF == 0) LOOKUP_FILL_NT16_B0(acc, a4, sel, cha, chb, nr, shift); else LOOKUP_FILL_NT16_B1(acc, a4, sel, cha, chb, nr, shift);
+    } else if constexpr (NT == 32) {
+        if constexpr (BUF == 0) LOOKUP_FILL_NT32_B0(acc, a4, sel, cha, chb, nr, shift); else LOOKUP_FILL_NT32_B1(acc, a4, sel, cha, chb, nr, shift);
+    } else {
+        if constexpr (BUF == 0) LOOKUP_FILL_NT64_B0(acc, a4, sel, cha, chb, nr, shift); else LOOKUP_FILL_NT64_B1(acc, a4, sel, cha, chb, nr, shift);
     }
 }
 
@@ -99,21 +88,21 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
 
     // ---- lane constants ----
     const int c0 = lane & 7;
-    uint32_t choff[8];   // byte offset, inside an expanded row, of the chunk this lane reads at step s
+    // Step s of a pixel reads chunk c_s = (c0 + s) & 7 of the expanded row of one activation code: the lanes
+    // of a wavefront touch eight different chunks per instruction whatever the codes are.  The chunk holds
+    // slots 8*c_s .. 8*c_s+7, i.e. input channel kk_s = c_s >> LOG_SETS of the fill, column group
+    // c_s & (SETS - 1).  The address (row << 8 | buffer << 7 | c_s << 4) is one v_perm_b32 of the
+    // activation dword and the packed chunk offsets: byte 1 <- activation byte kk_s, byte 0 <- offset byte.
+    uint32_t sel[8];
+    uint32_t cha = 0;
 #pragma unroll
-    for (int s = 0; s < 8; ++s)
-        choff[s] = (uint32_t)((c0 + s) & 7) << 4;
-    // The chunk of step s belongs to input channel kk_s = ((c0 + s) & 7) >> LOG_SETS of the fill.
-    // KS == 4: kk_s = (kk0 + ((p0 + s) >> 1)) & 3 with kk0 = c0 >> 1, p0 = c0 & 1, so after rotating the
-    //          activation dword right by kk0 bytes (and by p0 more for odd s) the byte index is the
-    //          compile-time constant s >> 1.
-    // KS == 2: kk_s is one bit, kept as a per-step lane mask in SGPRs.
-    const uint32_t rot_kk0 = (uint32_t)(c0 >> 1) << 3;
-    const uint32_t rot_p0 = (uint32_t)(c0 & 1) << 3;
-    uint64_t kk_mask[8];
-#pragma unroll
-    for (int s = 0; s < 8; ++s)
-        kk_mask[s] = __ballot(((((c0 + s) & 7) >> LOG_SETS) & 1) != 0);
+    for (int s = 0; s < 8; ++s) {
+        const uint32_t c = (uint32_t)(c0 + s) & 7u;
+        sel[s] = 0x0c0c0000u | ((4u + (c >> LOG_SETS)) << 8) | (uint32_t)(s & 3);
+        if (s < 4)
+            cha |= (c << 4) << (8 * s);
+    }
+    const uint32_t chb = cha ^ 0x40404040u; // (c0 + s + 4) & 7 == ((c0 + s) & 7) ^ 4
     // derive: item i of this lane transposes activation codes 4*lane .. 4*lane+3 of the staged table rows of
     // slots 4*jq_i .. 4*jq_i+3; the row permutation phys_row() and the rotation of jq by wavefront make
     // both the staged-row reads and the expanded-row writes bank-conflict free
@@ -122,7 +111,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     for (int i = 0; i < ITEMS; ++i)
         jq8[i] = (uint32_t)((lane + wave + i * kDenseWaves) & 15) * 8u; // byte offset of 4 slots in a row
     const uint32_t rd_lane = (uint32_t)lane * 8u;    // this lane's 8 bytes inside a staged 512-byte row
-    const uint32_t wr_row = (uint32_t)lane * 128u;
+    const uint32_t wr_row = (uint32_t)lane * 256u;   // expanded rows of the two buffers interleave: 256 bytes apart
     // staging: load j of this thread fetches 16 bytes of the table row of slot 16*j + tid/32
     const uint32_t st_slot = (uint32_t)tid >> 5;
     const uint32_t st_off = ((uint32_t)tid & 31u) * 16u;
@@ -147,15 +136,26 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         const int64_t row0 = (int64_t)rt * p.plan.rows_per_tile;
         const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
 
+        // ---- which wavefront-rows (64 consecutive output pixels) of the tile this wavefront owns ----
+        // The SIMD issues the older of its two wavefronts first, so the first four wavefronts get through
+        // their lookups faster; they own kOldShare/16 of the tile, and both halves reach the barrier together.
+        const int wrows = (int)((row_end - row0 + 63) / 64);
+        int wr_old = (wrows * kOldShare + 8) / 16;
+        wr_old = wr_old > 4 * R ? 4 * R : wr_old;
+        wr_old = wr_old < wrows - 4 * R ? wrows - 4 * R : wr_old;
+        const bool old_half = wave < kDenseWaves / 2;
+        const int wr_base = old_half ? wave : wr_old + wave - kDenseWaves / 2; // then every fourth wavefront-row
+        const int64_t wr_end = row0 + (int64_t)(old_half ? wr_old : wrows) * 64;
+
         // ---- per-pixel geometry (parked in LDS; only read back when the tap changes) ----
         bool rvalid[R];    // this lane's pixel exists
-        bool ractive[R];   // some lane of this wavefront has a pixel (wave-uniform)
+        uint32_t nr = 0;   // pixels of this lane whose wavefront row exists (a prefix; wave-uniform)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int64_t wrow = row0 + (int64_t)(r * kDenseWaves + wave) * 64;
-            ractive[r] = wrow < row_end;
+            const int64_t wrow = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
+            nr += (wrow < row_end && wrow < wr_end) ? 1u : 0u;
             const int64_t m = wrow + lane;
-            rvalid[r] = m < row_end;
+            rvalid[r] = m < row_end && wrow < wr_end;
             const int64_t mm = rvalid[r] ? m : row0;
             const int n = (int)(mm / ((int64_t)g.OH * g.OW));
             const int rem = (int)(mm - (int64_t)n * g.OH * g.OW);
@@ -248,7 +248,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 o[3].y = __builtin_amdgcn_perm(v[3].y, v[2].y, 0x07060302u);
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
-                    *reinterpret_cast<u32x2 *>(lds + buf * kExpandBytes + wr_row + jq8[i] + (uint32_t)k * (64u * 128u)) = o[k];
+                    *reinterpret_cast<u32x2 *>(lds + buf * 128u + wr_row + jq8[i] + (uint32_t)k * (64u * 256u)) = o[k];
             }
         };
 
@@ -276,25 +276,32 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         __syncthreads();
 
         // One phase: expand the next fill, stage the one after, issue the loads behind them, look up.
+        // The two wavefronts that share a SIMD do the expanding / staging at opposite ends of the phase, so
+        // that one of them always has lookups to issue while the other waits on LDS or on the memory pipeline.
+        const bool early = !old_half;
+        const uint32_t nr_s = __builtin_amdgcn_readfirstlane(nr);
         auto phase = [&](const int pcur, uint32_t (&act_cur)[R], uint32_t (&act_next)[R], auto buf_tag) {
             constexpr int BUF = decltype(buf_tag)::value;
-            const int sub = cur_sub; // sub-step of fill pcur inside its channel quad
-            // 1. consume what earlier phases loaded (nothing here waits on a fresh load)
-            if (pcur + 1 < fills)
-                derive(BUF ^ 1);          // fill pcur+1: staged rows -> expanded rows
-            if (pcur + 2 < fills)
-                store_stage(rows, BUF);   // fill pcur+2: registers -> staged rows (derive(pcur) read this buffer a phase ago)
-            __builtin_amdgcn_sched_barrier(0);
-            // 2. issue the loads later phases consume
-            if (pcur + 1 < fills) {
+            const uint32_t shift = (uint32_t)cur_sub * (32u / SUBS); // bits to rotate the channels of this fill down
+            auto feed = [&]() {
+                derive(BUF ^ 1);              // fill pcur+1: staged rows -> expanded rows
+                store_stage(rows, BUF);       // fill pcur+2: registers -> staged rows (read by derive a phase ago)
+                __builtin_amdgcn_sched_barrier(0);
                 load_rows(codes, rows);       // fill pcur+3
                 load_codes(pcur + 4, codes);
+            };
+            if (early)
+                feed();
+            __builtin_amdgcn_sched_barrier(0);
+            if (pcur + 1 < fills) {
                 advance_cursor();             // cursor -> fill pcur+1
                 load_acts(act_next);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // 3. look up
-            lookup_rows<NT, BUF>(acc, act_cur, sub, ractive, choff, rot_kk0, rot_p0, kk_mask);
+            lookup_fill<NT, BUF>(acc, act_cur, sel, cha, chb, nr_s, __builtin_amdgcn_readfirstlane(shift));
+            __builtin_amdgcn_sched_barrier(0);
+            if (!early)
+                feed();
             __syncthreads();
         };
         for (int pcur = 0; pcur < fills; pcur += 2) {
@@ -308,7 +315,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         for (int r = 0; r < R; ++r) {
             if (!rvalid[r])
                 continue;
-            const int64_t m = row0 + (int64_t)(r * kDenseWaves + wave) * 64 + lane;
+            const int64_t m = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64 + lane;
             // patch sum of the raw input in the reference's order (tap-major, channels ascending)
             const float psum = OUT_I32 ? 0.0f : p.psum[m];
             const float t1 = __fmul_rn(p.m2, psum);
