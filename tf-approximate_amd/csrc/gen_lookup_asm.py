@@ -1,110 +1,251 @@
 #!/usr/bin/env python3
-"""Generates lookup_asm.inc: the inline-assembly body of the LUT-GEMM lookup phase.
+"""Generates lookup_asm.inc: the inline-assembly body of one phase of the dense LUT-GEMM kernel.
 
     python gen_lookup_asm.py > lookup_asm.inc
 
-For each tile width NT (16, 32, 64 columns) and each of the two expanded-row buffers it emits one macro
+For each tile width NT (16, 32, 64 columns) and each parity BUF of the phase it emits one macro
+PHASE_NT<NT>_B<BUF>(...) that a wavefront executes once per fill p (BUF = p & 1), between two workgroup
+barriers.  The macro interleaves, in one instruction stream with hand-counted s_waitcnt:
 
-    LOOKUP_FILL_NT<NT>_B<buf>(ACC, A4, SEL, CHA, CHB, NR, SHIFT)
-
-that performs ALL lookups of one fill for the first NR (wave-uniform, 0..R) output pixels of the lane:
-
-  * a pixel needs eight 16-byte reads of the expanded row of its activation code.  The LDS address of step s
-    is ONE v_perm_b32: byte 1 <- the activation code (the rows of the two buffers interleave, so a row is
-    256 bytes apart from the next), byte 0 <- the lane's chunk offset for that step; SEL[s] is the lane's
-    byte selector, CHA / CHB hold the chunk offsets of steps 0-3 / 4-7;
-  * the reads run through a rolling window of eight that does not drain between pixels: as soon as chunk s
-    of pixel r has been accumulated its landing registers receive chunk s of pixel r + 1, so a wavefront
-    running alone on its SIMD still overlaps LDS latency with its adds;
-  * each arrived chunk is accumulated with eight v_add_u32_sdwa: one VALU op per table entry, the 16-bit
-    halves being picked by the SDWA source selector (no unpacking).  Step s accumulates into column group
-    s % (NT / 8);
-  * the buffer is selected by the instruction's immediate offset (128 bytes).
+  lookups   all lookups of fill p for the first NR (wave-uniform, 0..R) output pixels of the lane, out of
+            expanded-row buffer BUF.  A pixel needs eight 16-byte reads of the expanded row of its activation
+            code.  The LDS address of step s is ONE v_perm_b32 (byte 1 <- activation code: the rows of the two
+            buffers interleave, 256 bytes apart; byte 0 <- the lane's chunk offset).  The reads run through a
+            rolling window of eight that does not drain between pixels.  Each arrived chunk is accumulated
+            with eight v_add_u32_sdwa, one VALU op per table entry, the 16-bit halves being picked by the SDWA
+            source selector.  Step s accumulates into column group s % (NT / 8).
+  stage     the table rows of fill p+2 (in ROWS since the previous phase) go to staged-row buffer BUF.
+  loads     table rows of fill p+3 -> ROWS (addresses from CODES), filter codes of fill p+4 -> CODES,
+            activations of fill p+1 -> ANEXT; waited for at the end of the macro.
+  derive    the staged rows of fill p+1 (buffer BUF^1) are transposed into expanded-row buffer BUF^1: two
+            items per lane, each four 8-byte reads, eight v_perm_b32 and four 8-byte writes.
+            Stage, loads and derive are cut into micro-operations and one of them is slotted in behind every
+            16-byte chunk of the lookups, so that the memory pipeline and the LDS see them spread out instead
+            of as one burst per wavefront right after the barrier; what a wavefront with few pixels has not
+            placed by its last chunk follows behind it.
 
 NT = 16: a fill holds 4 input channels and the activation dword is used as it is.
 NT = 32 / 64: a fill holds 2 / 1 channels; the dword is first rotated right by SHIFT bits (an SGPR) so that
          the channels of this fill are its low bytes.
 
-The landing registers and the temporaries are fixed VGPRs declared as clobbers, because inline-asm operands
-cannot name the dwords of a 128-bit register tuple.
+LDS instructions complete in order, so "wait until operation X has completed" is s_waitcnt lgkmcnt(number
+of LDS operations issued after X); the generator keeps the issue queue and derives every count from it.
+The landing registers and temporaries are fixed VGPRs declared as clobbers, because inline-asm operands
+cannot name the dwords of a register tuple.
 """
 
+DERIVE_IN = 204            # 8 registers: four 8-byte staged-row reads of one derive item
+DERIVE_OUT = 212           # 6 registers: transposed dwords (two more reuse DERIVE_IN)
 ROT_TEMP = 218             # rotated activation dword of the pixel whose reads are being issued
+WR_TEMP = 219              # expanded-row write address of a derive item
 ADDR_BASE = 220            # 4 rolling address temporaries: v220..v223
 TEMP_BASE = 224            # 8 x 4 landing registers: v224..v255
-BUFFER_OFFSET = 128        # the rows of buffer 1 sit 128 bytes behind the rows of buffer 0
+CLOBBER_FIRST = DERIVE_IN
+
+
+class Stream:
+    """Instruction list plus the queue of LDS operations in flight."""
+
+    def __init__(self, lines=None, fifo=None, seq=0):
+        self.lines = lines if lines is not None else []
+        self.fifo = list(fifo) if fifo is not None else []
+        self.seq = seq
+
+    def fork(self):
+        return Stream(self.lines, self.fifo, self.seq + 100000)
+
+    def ins(self, text):
+        self.lines.append('"%s\\n\\t"' % text)
+
+    def label(self, text):
+        self.lines.append('"%s:\\n\\t"' % text)
+
+    def lds(self, text):
+        if len(self.fifo) == 15:     # lgkmcnt is a 4-bit counter: retire the oldest operation first
+            self.wait(self.fifo[0])
+        self.ins(text)
+        self.seq += 1
+        self.fifo.append(self.seq)
+        return self.seq
+
+    def wait(self, op):
+        """Wait until LDS operation `op` (and everything older) has completed."""
+        if op not in self.fifo:
+            return
+        i = self.fifo.index(op)
+        self.ins("s_waitcnt lgkmcnt(%d)" % (len(self.fifo) - 1 - i))
+        del self.fifo[:i + 1]
+
+    def drain(self):
+        self.ins("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        self.fifo = []
 
 
 def emit(nt, buf):
     sets = nt // 8
     rows = 2 * (64 // nt)
-    lines = []
+    other = buf ^ 1
 
-    def ins(text):
-        lines.append('"%s\\n\\t"' % text)
-
-    def rotate(r):
-        """Prepare the perm source of pixel r; returns the operand text."""
+    def rotate(st, r):
         if nt == 16:
             return "%%[a%d]" % r
-        ins("v_alignbit_b32 v%d, %%[a%d], %%[a%d], %%[shift]" % (ROT_TEMP, r, r))
+        st.ins("v_alignbit_b32 v%d, %%[a%d], %%[a%d], %%[shift]" % (ROT_TEMP, r, r))
         return "v%d" % ROT_TEMP
 
-    def read(src, step):
+    def read(st, src, step):
         b = TEMP_BASE + 4 * step
         va = ADDR_BASE + (step % 4)
-        ins("v_perm_b32 v%d, %s, %%[%s], %%[s%d]" % (va, src, "cha" if step < 4 else "chb", step))
-        off = " offset:%d" % (buf * BUFFER_OFFSET) if buf else ""
-        ins("ds_read_b128 v[%d:%d], v%d%s" % (b, b + 3, va, off))
+        st.ins("v_perm_b32 v%d, %s, %%[%s], %%[s%d]" % (va, src, "cha" if step < 4 else "chb", step))
+        off = " offset:128" if buf else ""
+        return st.lds("ds_read_b128 v[%d:%d], v%d%s" % (b, b + 3, va, off))
 
-    def adds(r, step):
+    def adds(st, r, step):
         b = TEMP_BASE + 4 * step
-        st = step % sets
+        g = step % sets
         for e in range(8):
-            reg = b + e // 2
-            sel = "WORD_0" if e % 2 == 0 else "WORD_1"
-            c = "%%[c%d_%d]" % (r, st * 8 + e)
-            ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:%s"
-                % (c, c, reg, sel))
+            c = "%%[c%d_%d]" % (r, g * 8 + e)
+            st.ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:%s"
+                   % (c, c, b + e // 2, "WORD_0" if e % 2 == 0 else "WORD_1"))
 
-    def body_last(r):
+    def prime(st):
+        src = rotate(st, 0)
+        return [read(st, src, s) for s in range(8)]
+
+    def body(st, r, pending, with_next, state):
+        """Accumulate pixel r (its reads are `pending`); with_next: refill the window with pixel r + 1.
+        One auxiliary micro-operation is slotted in behind every chunk."""
+        nxt = []
+        src = rotate(st, r + 1) if with_next else None
         for s in range(8):
-            ins("s_waitcnt lgkmcnt(%d)" % (7 - s))
-            adds(r, s)
+            st.wait(pending[s])
+            adds(st, r, s)
+            if with_next:
+                nxt.append(read(st, src, s))
+            aux_step(st, state)
+        return nxt
 
-    ins("s_cmp_eq_u32 %[nr], 0")
-    ins("s_cbranch_scc1 Lend_%=")
-    src = rotate(0)
-    for s in range(8):
-        read(src, s)
-    for r in range(rows - 1):
-        ins("s_cmp_lt_u32 %d, %%[nr]" % (r + 1))
-        ins("s_cbranch_scc0 Llast%d_%%=" % r)
-        src = rotate(r + 1)
-        for s in range(8):
-            ins("s_waitcnt lgkmcnt(7)")
-            adds(r, s)
-            read(src, s)
-    body_last(rows - 1)
-    ins("s_branch Lend_%=")
-    for r in range(rows - 1):
-        lines.append('"Llast%d_%%=:\\n\\t"' % r)
-        body_last(r)
-        if r != rows - 2:
-            ins("s_branch Lend_%=")
-    lines.append('"Lend_%=:\\n\\t"')
+    # ---- auxiliary work, cut into micro-operations that are spread over the chunk slots ----
+    def stage_write(j):      # table rows of fill p+2: registers -> staged rows [buf]
+        return lambda st, state: st.lds("ds_write_b128 %%[sta], %%[w%d] offset:%d" % (j, j * 8192 + buf * 32768))
 
-    outs = ", ".join('[c%d_%d] "+v"(ACC[%d][%d])' % (r, i, r, i) for r in range(rows) for i in range(nt))
-    inp = ['[a%d] "v"(A4[%d])' % (r, r) for r in range(rows)]
+    def row_load(j):         # table rows of fill p+3 <- table[code][16 bytes of this lane]
+        def f(st, state):
+            t = ADDR_BASE + 3    # the lookup address of a step is consumed by the read right behind it
+            st.ins("v_lshlrev_b32 v%d, 9, %%[k%d]" % (t, j))
+            st.ins("v_and_or_b32 v%d, v%d, %%[cmask], %%[sto]" % (t, t))
+            st.ins("buffer_load_dwordx4 %%[w%d], v%d, %%[tab], 0 offen" % (j, t))
+            st.ins("s_nop 0")
+        return f
+
+    def code_load(j):        # filter codes of fill p+4
+        return lambda st, state: st.ins("buffer_load_ushort %%[k%d], %%[cvo], %%[wq], %%[cso] offen offset:%d" % (j, 32 * j))
+
+    def act_load(r):         # activations of fill p+1
+        return lambda st, state: st.ins("buffer_load_dword %%[n%d], %%[t%d], %%[xq], %%[qoff] offen" % (r, r))
+
+    def derive_reads(item):
+        def f(st, state):
+            o = 64 * other  # staged-row buffer [other], in units of 512 bytes
+            st.lds("ds_read2st64_b64 v[%d:%d], %%[rd%d] offset0:%d offset1:%d"
+                   % (DERIVE_IN, DERIVE_IN + 3, item, o, o + 1))
+            state["dr"] = st.lds("ds_read2st64_b64 v[%d:%d], %%[rd%d] offset0:%d offset1:%d"
+                                 % (DERIVE_IN + 4, DERIVE_IN + 7, item, o + 2, o + 3))
+        return f
+
+    def derive_consume(item):
+        def f(st, state):
+            i, o = DERIVE_IN, DERIVE_OUT
+            st.wait(state["dr"])
+            # in: v[i:i+1] slot 0, v[i+2:i+3] slot 1, v[i+4:i+5] slot 2, v[i+6:i+7] slot 3 (two codes per dword)
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[plo]" % (o + 0, i + 2, i + 0))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[plo]" % (o + 1, i + 6, i + 4))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[phi]" % (o + 2, i + 2, i + 0))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[phi]" % (o + 3, i + 6, i + 4))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[plo]" % (o + 4, i + 3, i + 1))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[plo]" % (o + 5, i + 7, i + 5))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[phi]" % (i + 0, i + 3, i + 1))
+            st.ins("v_perm_b32 v%d, v%d, v%d, %%[phi]" % (i + 1, i + 7, i + 5))
+            if other:
+                st.ins("v_add_u32 v%d, 128, %%[wr%d]" % (WR_TEMP, item))
+                wa = "v%d" % WR_TEMP
+            else:
+                wa = "%%[wr%d]" % item
+            st.lds("ds_write2st64_b64 %s, v[%d:%d], v[%d:%d] offset0:0 offset1:32" % (wa, o, o + 1, o + 2, o + 3))
+            st.lds("ds_write2st64_b64 %s, v[%d:%d], v[%d:%d] offset0:64 offset1:96" % (wa, o + 4, o + 5, i, i + 1))
+        return f
+
+    def both(f, g):
+        return lambda st, state: (f(st, state), g(st, state))
+
+    # reads of a derive item are issued nine slots before its transposes
+    aux = [derive_reads(0)]
+    for j in range(4):
+        aux += [stage_write(j), row_load(j)]
+    aux += [both(derive_consume(0), derive_reads(1))]
+    aux += [code_load(j) for j in range(4)]
+    aux += [both(act_load(r), act_load(r + 1)) for r in range(0, rows, 2)]
+    while len(aux) < 18:
+        aux.append(lambda st, state: None)
+    aux += [derive_consume(1)]
+
+    def aux_step(st, state):
+        if state["pos"] < len(aux):
+            aux[state["pos"]](st, state)
+            state["pos"] += 1
+
+    def aux_rest(st, state):
+        while state["pos"] < len(aux):
+            aux_step(st, state)
+
+    main = Stream()
+    main.ins("s_cmp_eq_u32 %[nr], 0")
+    main.ins("s_cbranch_scc1 Lzero_%=")
+    pending = prime(main)
+    state = {"pos": 0, "dr": None}
+    forks = []
+    for r in range(rows):
+        if r < rows - 1:
+            main.ins("s_cmp_lt_u32 %d, %%[nr]" % (r + 1))
+            main.ins("s_cbranch_scc0 Llast%d_%%=" % r)
+            forks.append((r, main.fork(), list(pending), dict(state)))
+            pending = body(main, r, pending, True, state)
+        else:
+            body(main, r, pending, False, state)
+    aux_rest(main, state)
+    main.drain()
+    main.ins("s_branch Lend_%=")
+    for r, st, pend, stt in forks:
+        st.label("Llast%d_%%=" % r)
+        body(st, r, pend, False, stt)
+        aux_rest(st, stt)
+        st.drain()
+        st.ins("s_branch Lend_%=")
+    zero = Stream(main.lines)
+    zero.label("Lzero_%=")
+    aux_rest(zero, {"pos": 0, "dr": None})
+    zero.drain()
+    zero.label("Lend_%=")
+
+    outs = ['[c%d_%d] "+v"(ACC[%d][%d])' % (r, i, r, i) for r in range(rows) for i in range(nt)]
+    outs += ['[w%d] "+v"(ROWS[%d])' % (j, j) for j in range(4)]
+    outs += ['[k%d] "+v"(CODES[%d])' % (j, j) for j in range(4)]
+    outs += ['[n%d] "=&v"(ANEXT[%d])' % (r, r) for r in range(rows)]
+    inp = ['[a%d] "v"(ACUR[%d])' % (r, r) for r in range(rows)]
+    inp += ['[t%d] "v"(TAPOFF[%d])' % (r, r) for r in range(rows)]
     inp += ['[s%d] "v"(SEL[%d])' % (i, i) for i in range(8)]
     inp += ['[cha] "v"(CHA)', '[chb] "v"(CHB)', '[nr] "s"(NR)']
+    inp += ['[sta] "v"(STA)', '[sto] "v"(STO)', '[cvo] "v"(CVO)']
+    inp += ['[rd0] "v"(RD[0])', '[rd1] "v"(RD[1])', '[wr0] "v"(WR[0])', '[wr1] "v"(WR[1])']
+    inp += ['[plo] "s"(0x05040100u)', '[phi] "s"(0x07060302u)', '[cmask] "s"(0x01fffe00u)']
+    inp += ['[tab] "s"(TAB)', '[wq] "s"(WQ)', '[xq] "s"(XQ)', '[cso] "s"(CSO)', '[qoff] "s"(QOFF)']
     if nt != 16:
         inp.append('[shift] "s"(SHIFT)')
-    clob = ", ".join('"v%d"' % r for r in [ROT_TEMP] + list(range(ADDR_BASE, TEMP_BASE + 32)))
-    body = " \\\n        ".join(lines)
-    return ("#define LOOKUP_FILL_NT%d_B%d(ACC, A4, SEL, CHA, CHB, NR, SHIFT) \\\n    asm volatile( \\\n        %s \\\n"
+    clob = ", ".join('"v%d"' % r for r in range(CLOBBER_FIRST, TEMP_BASE + 32))
+    body_text = " \\\n        ".join(main.lines)
+    args = "ACC, ACUR, ANEXT, TAPOFF, ROWS, CODES, SEL, CHA, CHB, NR, SHIFT, STA, STO, CVO, RD, WR, TAB, WQ, XQ, CSO, QOFF"
+    return ("#define PHASE_NT%d_B%d(%s) \\\n    asm volatile( \\\n        %s \\\n"
             "        : %s \\\n        : %s \\\n        : %s, \"scc\", \"memory\")\n"
-            % (nt, buf, body, outs, ", ".join(inp), clob))
+            % (nt, buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))
 
 
 if __name__ == "__main__":

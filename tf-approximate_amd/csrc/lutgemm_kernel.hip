@@ -59,18 +59,35 @@ struct DenseCfg {
     static constexpr int SUBS = 4 / KS;       // fills per channel quad
 };
 
-// Lookups of one fill for the first nr output pixels of this lane (out of expanded-row buffer BUF).
+// Lane constants of the phase body.
+struct PhaseConsts {
+    uint32_t sel[8];   // v_perm_b32 selectors that build the lookup address of step s
+    uint32_t cha, chb; // packed chunk offsets of steps 0-3 / 4-7
+    uint32_t sta;      // LDS address of this thread's 16 bytes in staged row (thread / 32) of buffer 0
+    uint32_t sto;      // byte offset of those 16 bytes inside a 512-byte table row
+    uint32_t cvo;      // byte offset of filter code (thread / 32) inside the 64 codes of a fill
+    uint32_t rd[2];    // LDS address (buffer 0) of the staged-row bytes derive item i reads
+    uint32_t wr[2];    // LDS address (buffer 0) of the expanded-row bytes derive item i writes
+};
+
+// One phase (see gen_lookup_asm.py): lookups of fill p out of expanded-row buffer BUF, interleaved with staging
+// the rows of fill p+2, loading rows / codes / activations of later fills and expanding fill p+1.
 template <int NT, int BUF>
-__device__ __forceinline__ void lookup_fill(int32_t (&acc)[DenseCfg<NT>::R][NT], const uint32_t (&a4)[DenseCfg<NT>::R],
-                                            const uint32_t (&sel)[8], const uint32_t cha, const uint32_t chb,
-                                            const uint32_t nr, const uint32_t shift)
+__device__ __forceinline__ void phase_body(int32_t (&acc)[DenseCfg<NT>::R][NT], const uint32_t (&acur)[DenseCfg<NT>::R],
+                                           uint32_t (&anext)[DenseCfg<NT>::R], const uint32_t (&tapoff)[DenseCfg<NT>::R],
+                                           u32x4 (&rows)[4], uint32_t (&codes)[4], const PhaseConsts &k,
+                                           const uint32_t nr, const uint32_t shift, const rsrc_t tab, const rsrc_t wq,
+                                           const rsrc_t xq, const uint32_t cso, const uint32_t qoff)
 {
     if constexpr (NT == 16) {
-        if constexpr (BUF == 0) LOOKUP_FILL_NT16_B0(acc, a4, sel, cha, chb, nr, shift); else LOOKUP_FILL_NT16_B1(acc, a4, sel, cha, chb, nr, shift);
+        if constexpr (BUF == 0) PHASE_NT16_B0(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        else PHASE_NT16_B1(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
     } else if constexpr (NT == 32) {
-        if constexpr (BUF == 0) LOOKUP_FILL_NT32_B0(acc, a4, sel, cha, chb, nr, shift); else LOOKUP_FILL_NT32_B1(acc, a4, sel, cha, chb, nr, shift);
+        if constexpr (BUF == 0) PHASE_NT32_B0(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        else PHASE_NT32_B1(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
     } else {
-        if constexpr (BUF == 0) LOOKUP_FILL_NT64_B0(acc, a4, sel, cha, chb, nr, shift); else LOOKUP_FILL_NT64_B1(acc, a4, sel, cha, chb, nr, shift);
+        if constexpr (BUF == 0) PHASE_NT64_B0(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        else PHASE_NT64_B1(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
     }
 }
 
@@ -275,33 +292,38 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         load_codes(3, codes);
         __syncthreads();
 
-        // One phase: expand the next fill, stage the one after, issue the loads behind them, look up.
-        // The two wavefronts that share a SIMD do the expanding / staging at opposite ends of the phase, so
-        // that one of them always has lookups to issue while the other waits on LDS or on the memory pipeline.
-        const bool early = !old_half;
+        // One phase per fill, one barrier per phase.
+        PhaseConsts k;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            k.sel[i] = sel[i];
+        k.cha = cha;
+        k.chb = chb;
+        k.sta = 2u * kExpandBytes + st_slot * 512u + st_off;
+        k.sto = st_off;
+        k.cvo = st_slot * 2u;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            k.rd[i] = 2u * kExpandBytes + (jq8[i] / 2u) * 512u + rd_lane;
+            k.wr[i] = wr_row + jq8[i];
+        }
         const uint32_t nr_s = __builtin_amdgcn_readfirstlane(nr);
+        // Entering phase p the activation cursor stands on fill p+1 and shift_cur belongs to fill p; the cursor
+        // is moved on behind the phase body, where most wavefronts would otherwise only wait for the barrier.
+        uint32_t shift_cur = 0;
+        if (fills > 1)
+            advance_cursor();
         auto phase = [&](const int pcur, uint32_t (&act_cur)[R], uint32_t (&act_next)[R], auto buf_tag) {
             constexpr int BUF = decltype(buf_tag)::value;
-            const uint32_t shift = (uint32_t)cur_sub * (32u / SUBS); // bits to rotate the channels of this fill down
-            auto feed = [&]() {
-                derive(BUF ^ 1);              // fill pcur+1: staged rows -> expanded rows
-                store_stage(rows, BUF);       // fill pcur+2: registers -> staged rows (read by derive a phase ago)
-                __builtin_amdgcn_sched_barrier(0);
-                load_rows(codes, rows);       // fill pcur+3
-                load_codes(pcur + 4, codes);
-            };
-            if (early)
-                feed();
-            __builtin_amdgcn_sched_barrier(0);
-            if (pcur + 1 < fills) {
-                advance_cursor();             // cursor -> fill pcur+1
-                load_acts(act_next);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            lookup_fill<NT, BUF>(acc, act_cur, sel, cha, chb, nr_s, __builtin_amdgcn_readfirstlane(shift));
-            __builtin_amdgcn_sched_barrier(0);
-            if (!early)
-                feed();
+            const int fcodes = pcur + 4 < fills ? pcur + 4 : fills - 1;
+            const uint32_t cso = wq_tile + (uint32_t)fcodes * 128u;
+            const uint32_t qoff = (uint32_t)(cur_q * g.W * 4);
+            phase_body<NT, BUF>(acc, act_cur, act_next, idx_tap, rows, codes, k, nr_s,
+                                __builtin_amdgcn_readfirstlane(shift_cur), tab_rsrc, wq_rsrc, xq_rsrc,
+                                __builtin_amdgcn_readfirstlane(cso), __builtin_amdgcn_readfirstlane(qoff));
+            shift_cur = (uint32_t)cur_sub * (32u / SUBS); // bits to rotate the channels of fill pcur+1 down
+            if (pcur + 2 < fills)
+                advance_cursor();             // -> fill pcur+2 (re-reads the parked geometry on a new tap)
             __syncthreads();
         };
         for (int pcur = 0; pcur < fills; pcur += 2) {
