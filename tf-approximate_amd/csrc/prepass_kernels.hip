@@ -104,63 +104,156 @@ __global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict
 }
 
 // Patch sums for C % 4 == 0, same order and same results as patch_sums_kernel.  One thread per output
-// pixel still owns the sequential chain, but the floats arrive through LDS: for each tap the block loads
-// the 256 input pixels of its 256 output pixels cooperatively (8 lanes read the 128 contiguous bytes of a
-// 32-channel slice of one pixel), so a wavefront touches 8 memory lines per load instead of 64.
+// pixel still owns the sequential chain, but the floats arrive through LDS: for each tap and 32-channel
+// slice the block loads the 256 input pixels of its 256 output pixels cooperatively (8 lanes read the 128
+// contiguous bytes of one pixel's slice), so a wavefront touches 8 memory lines per load instead of 64.
+// The loads of the next slice are in flight while the block adds up the current one.
 constexpr int kPsTile = 256;  // output pixels per block
 constexpr int kPsCh = 32;     // channels per LDS slice
 constexpr int kPsRow = kPsCh + 4; // padded row (floats): conflict-free 16-byte accesses
+constexpr int kPsLoads = kPsCh / 4 * kPsTile / kPsTile; // float4 loads per thread per slice
 
 __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *__restrict__ x, ConvGeom g,
                                                                     float *__restrict__ psum)
 {
-    __shared__ int64_t bases[kPsTile];
+    __shared__ int pix_base[kPsTile];  // (n * H) of the pixel's image, or -1 when the pixel does not exist
+    __shared__ int pix_hw[kPsTile];    // input row / column of tap (0, 0), 16 bits each
     __shared__ __align__(16) float tile[kPsTile * kPsRow];
+    constexpr int kQuads = kPsCh / 4;  // float4 per pixel per slice
     const int t = threadIdx.x;
     const int64_t m = (int64_t)blockIdx.x * kPsTile + t;
     const bool valid = m < g.M;
-    int n = 0, ih0 = 0, iw0 = 0;
-    if (valid) {
-        n = (int)(m / ((int64_t)g.OH * g.OW));
-        const int rem = (int)(m - (int64_t)n * g.OH * g.OW);
-        const int oh = rem / g.OW, ow = rem - oh * g.OW;
-        ih0 = oh * g.sh - g.ph;
-        iw0 = ow * g.sw - g.pw;
-    }
-    float s = 0.0f;
-    constexpr int kQuads = kPsCh / 4;                       // float4 per pixel per slice
-    constexpr int kLoads = kPsTile * kQuads / kPsTile;      // float4 loads per thread per slice
-    for (int kh = 0; kh < g.KH; ++kh)
-        for (int kw = 0; kw < g.KW; ++kw) {
-            const int ih = ih0 + kh * g.dh, iw = iw0 + kw * g.dw;
-            const bool inb = valid && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-            __syncthreads(); // previous slice consumed
-            bases[t] = inb ? (((int64_t)n * g.H + ih) * g.W + iw) * g.C : (int64_t)-1;
-            for (int c0 = 0; c0 < g.C; c0 += kPsCh) {
-                __syncthreads(); // bases visible / previous slice consumed
-#pragma unroll
-                for (int i = 0; i < kLoads; ++i) {
-                    const int idx = t + i * kPsTile;
-                    const int pl = idx / kQuads, j = idx % kQuads;
-                    const int64_t b = bases[pl];
-                    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                    if (b >= 0 && c0 + j * 4 < g.C)
-                        v = *reinterpret_cast<const float4 *>(x + b + c0 + j * 4);
-                    *reinterpret_cast<float4 *>(&tile[pl * kPsRow + j * 4]) = v;
-                }
-                __syncthreads();
-                const int nq = (g.C - c0 < kPsCh ? g.C - c0 : kPsCh) / 4;
-                for (int j = 0; j < nq; ++j) {
-                    const float4 v = *reinterpret_cast<const float4 *>(&tile[t * kPsRow + j * 4]);
-                    s = __fadd_rn(s, v.x);
-                    s = __fadd_rn(s, v.y);
-                    s = __fadd_rn(s, v.z);
-                    s = __fadd_rn(s, v.w);
-                }
-            }
+    {
+        int n = 0, ih0 = 0, iw0 = 0;
+        if (valid) {
+            n = (int)(m / ((int64_t)g.OH * g.OW));
+            const int rem = (int)(m - (int64_t)n * g.OH * g.OW);
+            const int oh = rem / g.OW, ow = rem - oh * g.OW;
+            ih0 = oh * g.sh - g.ph;
+            iw0 = ow * g.sw - g.pw;
         }
+        pix_base[t] = valid ? n * g.H : -1;
+        pix_hw[t] = (ih0 << 16) | (iw0 & 0xffff);
+    }
+    __syncthreads();
+    // this thread fetches quad j of the pixels pl0, pl0 + 32, ... of every slice
+    const int j = t % kQuads, pl0 = t / kQuads;
+    int lbase[kPsLoads], lih[kPsLoads], liw[kPsLoads];
+#pragma unroll
+    for (int i = 0; i < kPsLoads; ++i) {
+        const int pl = pl0 + i * (kPsTile / kQuads);
+        lbase[i] = pix_base[pl];
+        lih[i] = pix_hw[pl] >> 16;
+        liw[i] = (int)(int16_t)(pix_hw[pl] & 0xffff);
+    }
+    const int slices = (g.C + kPsCh - 1) / kPsCh;
+    const int iters = g.KH * g.KW * slices;
+    float4 v[kPsLoads];
+    auto fetch = [&](int it) {
+        const int tap = it / slices, c0 = (it - tap * slices) * kPsCh;
+        const int kh = tap / g.KW, kw = tap - kh * g.KW;
+#pragma unroll
+        for (int i = 0; i < kPsLoads; ++i) {
+            const int ih = lih[i] + kh * g.dh, iw = liw[i] + kw * g.dw;
+            v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (lbase[i] >= 0 && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && c0 + j * 4 < g.C)
+                v[i] = *reinterpret_cast<const float4 *>(x + ((int64_t)(lbase[i] + ih) * g.W + iw) * g.C + c0 + j * 4);
+        }
+    };
+    float s = 0.0f;
+    fetch(0);
+    for (int it = 0; it < iters; ++it) {
+        __syncthreads(); // previous slice consumed
+#pragma unroll
+        for (int i = 0; i < kPsLoads; ++i)
+            *reinterpret_cast<float4 *>(&tile[(pl0 + i * (kPsTile / kQuads)) * kPsRow + j * 4]) = v[i];
+        __syncthreads();
+        if (it + 1 < iters)
+            fetch(it + 1);
+        const int c0 = (it % slices) * kPsCh;
+        const int nq = (g.C - c0 < kPsCh ? g.C - c0 : kPsCh) / 4;
+        // taps outside the image were stored as 0.0f: x + 0.0f == x (the sum never is -0.0f after a real term,
+        // and 0.0f + 0.0f stays +0.0f as in the reference, which starts from +0.0f)
+        for (int q = 0; q < nq; ++q) {
+            const float4 w = *reinterpret_cast<const float4 *>(&tile[t * kPsRow + q * 4]);
+            s = __fadd_rn(s, w.x);
+            s = __fadd_rn(s, w.y);
+            s = __fadd_rn(s, w.z);
+            s = __fadd_rn(s, w.w);
+        }
+    }
     if (valid)
         psum[m] = s;
+}
+
+// Patch sums for C % 4 == 0 when the input rows under a band of output rows fit in LDS: same order and same
+// results as patch_sums_kernel.  A block owns `rb` consecutive output rows of one image (one thread per output
+// pixel) and first copies the input rows they touch into LDS, so every input float is fetched from memory
+// about once (plus the halo) instead of once per filter tap; the sequential chains then read LDS only.
+// Pixels are padded to C + 4 floats so that the 16-byte reads of neighbouring threads fall into different banks.
+__global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, ConvGeom g, int rb,
+                                                                int in_rows, float *__restrict__ psum)
+{
+    extern __shared__ __align__(16) unsigned char ps_lds[];
+    float *const rows = reinterpret_cast<float *>(ps_lds);
+    const int t = threadIdx.x;
+    const int bands = (g.OH + rb - 1) / rb;
+    const int n = blockIdx.x / bands;
+    const int oh0 = (blockIdx.x - n * bands) * rb;
+    const int ih_first = oh0 * g.sh - g.ph;  // input row held in LDS row 0 (may lie outside the image)
+    const int pitch = g.C + 4;
+    if (blockDim.x % g.C4 == 0) {
+        // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns
+        const int q = t % g.C4, w0 = t / g.C4, wstep = blockDim.x / g.C4;
+        for (int r = 0; r < in_rows; ++r) {
+            const int ih = ih_first + r;
+            const bool inb = (unsigned)ih < (unsigned)g.H;
+            const float *src = x + (((int64_t)n * g.H + (inb ? ih : 0)) * g.W) * g.C + q * 4;
+            for (int w = w0; w < g.W; w += wstep) {
+                float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (inb)
+                    v = *reinterpret_cast<const float4 *>(src + (int64_t)w * g.C);
+                *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
+            }
+        }
+    } else {
+        const int quads_per_row = g.W * g.C4;
+        const int total = in_rows * quads_per_row;
+        for (int i = t; i < total; i += blockDim.x) {
+            const int r = i / quads_per_row, rem = i - r * quads_per_row;
+            const int w = rem / g.C4, q = rem - w * g.C4;
+            const int ih = ih_first + r;
+            float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if ((unsigned)ih < (unsigned)g.H)
+                v = *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + w) * g.C + q * 4);
+            *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
+        }
+    }
+    __syncthreads();
+    const int ohl = t / g.OW, ow = t - ohl * g.OW;
+    const int oh = oh0 + ohl;
+    if (ohl >= rb || oh >= g.OH)
+        return;
+    const int iw0 = ow * g.sw - g.pw;
+    float s = 0.0f;
+    for (int kh = 0; kh < g.KH; ++kh) {
+        const int r = ohl * g.sh + kh * g.dh;        // LDS row of this tap; rows outside the image hold zeros,
+        for (int kw = 0; kw < g.KW; ++kw) {          // and x + 0.0f == x, so they need no branch
+            const int iw = iw0 + kw * g.dw;
+            if ((unsigned)iw >= (unsigned)g.W)
+                continue;
+            const float *src = &rows[(r * g.W + iw) * pitch];
+#pragma unroll 8
+            for (int q = 0; q < g.C4; ++q) {
+                const float4 v = *reinterpret_cast<const float4 *>(src + q * 4);
+                s = __fadd_rn(s, v.x);
+                s = __fadd_rn(s, v.y);
+                s = __fadd_rn(s, v.z);
+                s = __fadd_rn(s, v.w);
+            }
+        }
+    }
+    psum[((int64_t)n * g.OH + oh) * g.OW + ow] = s;
 }
 
 // Same relayout for caller-supplied codes (uint8 NHWC).
@@ -223,31 +316,47 @@ __global__ void __launch_bounds__(256) filter_pack_kernel(const float *__restric
 
 // Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one thread per output column,
 // rows (h, w, c) ascending.
-// A block owns 64 columns; all 256 threads stage 128 filter rows at a time into LDS (coalesced, many loads in
-// flight), then the first 64 threads extend their column's sequential sum from LDS.
-__global__ void __launch_bounds__(256) filter_sums_kernel(const float *__restrict__ filter, int K, int Co,
-                                                           float *__restrict__ fsum)
+// A block owns 64 columns; all 1024 threads stage up to 512 filter rows at a time into LDS (coalesced, every
+// load of a pass in flight at once), then the first 64 threads extend their column's sequential sum from LDS,
+// 32 independent LDS reads ahead of the dependent chain of adds.
+constexpr int kFsRows = 512, kFsThreads = 1024;
+constexpr int kFsLdsBytes = kFsRows * 65 * 4;
+
+__global__ void __launch_bounds__(kFsThreads) filter_sums_kernel(const float *__restrict__ filter, int K, int Co,
+                                                                  float *__restrict__ fsum)
 {
-    constexpr int kRows = 128;
-    __shared__ float stage[kRows * 65];
+    constexpr int kBatch = 32, kPer = kFsRows * 64 / kFsThreads; // loads per thread per pass
+    extern __shared__ __align__(16) unsigned char fs_lds[];
+    float *const stage = reinterpret_cast<float *>(fs_lds);
     const int col0 = blockIdx.x * 64;
     const int t = threadIdx.x;
-    const int cl = t & 63, rsub = t >> 6; // 4 rows per pass
+    const int cl = t & 63, rsub = t >> 6; // 16 rows per step
     float s = 0.0f;
-    for (int k0 = 0; k0 < K; k0 += kRows) {
-        __syncthreads();
-#pragma unroll 8
-        for (int r = rsub; r < kRows; r += 4) {
-            const int k = k0 + r;
-            float v = 0.0f;
-            if (k < K && col0 + cl < Co)
-                v = filter[(int64_t)k * Co + col0 + cl];
-            stage[r * 65 + cl] = v;
+    for (int k0 = 0; k0 < K; k0 += kFsRows) {
+        float v[kPer];
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int k = k0 + rsub + i * (kFsThreads / 64);
+            v[i] = (k < K && col0 + cl < Co) ? filter[(int64_t)k * Co + col0 + cl] : 0.0f;
         }
+        __syncthreads(); // previous pass consumed
+#pragma unroll
+        for (int i = 0; i < kPer; ++i)
+            stage[(rsub + i * (kFsThreads / 64)) * 65 + cl] = v[i];
         __syncthreads();
         if (t < 64) {
-            const int nr = (K - k0 < kRows) ? K - k0 : kRows;
-            for (int r = 0; r < nr; ++r)
+            const int nr = (K - k0 < kFsRows) ? K - k0 : kFsRows;
+            int r = 0;
+            for (; r + kBatch <= nr; r += kBatch) {
+                float w[kBatch];
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i)
+                    w[i] = stage[(r + i) * 65 + t];
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i)
+                    s = __fadd_rn(s, w[i]);
+            }
+            for (; r < nr; ++r)
                 s = __fadd_rn(s, stage[r * 65 + t]);
         }
     }
@@ -321,7 +430,36 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float off
 
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream)
 {
-    if ((g.C & 3) == 0 && ((uintptr_t)x & 15) == 0)
+    const bool vec = (g.C & 3) == 0 && ((uintptr_t)x & 15) == 0;
+    if (vec && g.OW <= 1024) {
+        // largest band of output rows whose input rows fit in 96 KiB of LDS and whose pixels fit in one block,
+        // but no larger than what still leaves every CU a few blocks
+        const int64_t row_bytes = (int64_t)g.W * (g.C + 4) * 4;
+        int rb = 0, in_rows = 0;
+        for (int cand = 1; cand <= g.OH && cand * g.OW <= 1024; ++cand) {
+            const int rows_needed = (cand - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+            if (rows_needed * row_bytes > 96 * 1024)
+                break;
+            if (cand > 1 && (int64_t)g.N * ((g.OH + cand - 1) / cand) < 1024)
+                break;
+            rb = cand;
+            in_rows = rows_needed;
+        }
+        if (rb > 0) {
+            int threads = ((rb * g.OW + 63) / 64) * 64;
+            threads = threads < 512 ? 512 : threads;   // the copy into LDS wants more threads than there are pixels
+            const size_t lds = (size_t)in_rows * row_bytes;
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(patch_sums_rows_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            if (e != hipSuccess)
+                return e;
+            const int bands = (g.OH + rb - 1) / rb;
+            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(g.N * bands)), dim3(threads), lds, stream, x, g,
+                               rb, in_rows, psum);
+            return hipGetLastError();
+        }
+    }
+    if (vec)
         hipLaunchKernelGGL(patch_sums_tiled_kernel, dim3(blocks_for(g.M, kPsTile)), dim3(kPsTile), 0, stream, x, g,
                            psum);
     else
@@ -352,7 +490,11 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !fsum || !filter)
         return e;
-    hipLaunchKernelGGL(filter_sums_kernel, dim3(blocks_for(g.Co, 64)), dim3(256), 0, stream, filter, g.K, g.Co,
+    hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(filter_sums_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kFsLdsBytes);
+    if (ea != hipSuccess)
+        return ea;
+    hipLaunchKernelGGL(filter_sums_kernel, dim3(blocks_for(g.Co, 64)), dim3(kFsThreads), kFsLdsBytes, stream, filter, g.K, g.Co,
                        fsum);
     return hipGetLastError();
 }
