@@ -36,7 +36,26 @@ def build(verbose=False, extra=()):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+    build_harness(verbose)
     return LIB
+
+
+SHELL = os.path.join(HERE, "shell")
+HARNESS = os.path.join(HERE, "axconv_harness")
+
+
+def build_harness(verbose=False):
+    """The TensorFlow-free op shell plus the standalone C++ harness, linked against the library."""
+    cmd = ["hipcc", "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument",
+           "-I", os.path.join(ROOT, "include"), "-I", SHELL,
+           os.path.join(SHELL, "approx_conv2d_op.cc"), os.path.join(SHELL, "axconv_harness.cc"),
+           "-L", HERE, "-laxconv_hip", "-Wl,-rpath,$ORIGIN", "-o", HARNESS]
+    if verbose:
+        print(" ".join(cmd))
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed (harness):\n" + res.stdout)
+    return HARNESS
 
 
 if __name__ == "__main__":
