@@ -48,6 +48,9 @@ def main():
     ap.add_argument("--codes", default="uniform", choices=["uniform", "halfnormal"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="instead of the benchmark, run a plain device copy of MIB MiB five times: the known-size "
+                         "kernel that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no cross-GPU step (output pixels shard without "
@@ -55,6 +58,15 @@ def main():
 
     import numpy as np
     import torch
+    if args.copy_calibration:
+        n = args.copy_calibration * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": n * 4, "copy_calibration_bytes_written": n * 4, "launches": 5}))
+        return
     import __graft_entry__ as entry
     pkg = entry.load_package()
     from tf_approximate_amd import ops, synth

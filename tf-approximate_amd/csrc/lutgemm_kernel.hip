@@ -148,8 +148,21 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     (void)taps;
 
     for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int ct = tile % p.plan.n_col_tiles;
-        const int rt = tile / p.plan.n_col_tiles;
+        // Workgroups are handed to the 8 XCDs round-robin, and each XCD has its own L2.  The column tiles of one
+        // row tile read the same activations, so they go to the same XCD, next to each other in time:
+        // inside a group of 8 * n_col_tiles consecutive tiles, tile r is (row tile r % 8, column tile r / 8).
+        int ct, rt;
+        {
+            const int nct = p.plan.n_col_tiles, group = 8 * nct;
+            const int gi = tile / group, r = tile - gi * group;
+            if ((gi + 1) * group <= ntiles) {
+                ct = r >> 3;
+                rt = gi * 8 + (r & 7);
+            } else { // the ragged tail keeps the plain order
+                ct = tile % nct;
+                rt = tile / nct;
+            }
+        }
         const int64_t row0 = (int64_t)rt * p.plan.rows_per_tile;
         const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
 
@@ -345,20 +358,42 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             for (int set = 0; set < SETS; ++set) {
                 const int h = (c0 + set) & (SETS - 1);
                 const int col0 = ct * NT + h * 8;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int col = col0 + e;
-                    if (col >= g.Co)
-                        continue;
-                    const int32_t a = acc[r][set * 8 + e];
-                    if (OUT_I32) {
-                        p.out_i[m * g.Co + col] = a;
+                if (col0 >= g.Co)
+                    continue;
+                const int64_t o = m * g.Co + col0;
+                const bool vec = (g.Co & 3) == 0 && col0 + 8 <= g.Co; // 32 contiguous, 16-byte aligned bytes
+                if (OUT_I32) {
+                    if (vec) {
+                        typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+                        i32x4 lo = {acc[r][set * 8 + 0], acc[r][set * 8 + 1], acc[r][set * 8 + 2], acc[r][set * 8 + 3]};
+                        i32x4 hi = {acc[r][set * 8 + 4], acc[r][set * 8 + 5], acc[r][set * 8 + 6], acc[r][set * 8 + 7]};
+                        *reinterpret_cast<i32x4 *>(p.out_i + o) = lo;
+                        *reinterpret_cast<i32x4 *>(p.out_i + o + 4) = hi;
                     } else {
-                        const float t0 = __fmul_rn((float)a, p.s1xs2);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (col0 + e < g.Co)
+                                p.out_i[o + e] = acc[r][set * 8 + e];
+                    }
+                } else {
+                    float v[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int col = col0 + e < g.Co ? col0 + e : g.Co - 1;
+                        const float t0 = __fmul_rn((float)acc[r][set * 8 + e], p.s1xs2);
                         const float t2 = __fadd_rn(t0, t1);
                         const float t3 = __fmul_rn(p.m1, p.fsum[col]);
                         const float t4 = __fadd_rn(t2, t3);
-                        p.out_f[m * g.Co + col] = __fsub_rn(t4, p.k_m1xm2);
+                        v[e] = __fsub_rn(t4, p.k_m1xm2);
+                    }
+                    if (vec) {
+                        *reinterpret_cast<float4 *>(p.out_f + o) = make_float4(v[0], v[1], v[2], v[3]);
+                        *reinterpret_cast<float4 *>(p.out_f + o + 4) = make_float4(v[4], v[5], v[6], v[7]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (col0 + e < g.Co)
+                                p.out_f[o + e] = v[e];
                     }
                 }
             }
