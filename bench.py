@@ -38,6 +38,12 @@ WORKLOADS = {
 }
 DEFAULT = "conv3x3_b64_56x56x64_to_64_s1_same"
 
+# HBM bytes per launch of the main kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
+# scaled by what the same counter reads for --copy-calibration (profiles/lutgemm_expand_conv3x3_b64_56x56x64.md).
+MEASURED_TRAFFIC_BYTES = {
+    "conv3x3_b64_56x56x64_to_64_s1_same": 2.000 * 9384.8 * 1024 + 1.000 * 61865.1 * 1024,
+}
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -131,7 +137,7 @@ def main():
         "peak": round(peak / 1e9, 1),
         "unit": "Glookup/s",
         "frac": round(achieved / peak, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
         "kernel_ms": round(main_ms, 4),
         "lookups_per_launch": lookups,
         "peak_nominal": round(NOMINAL_LDS_LOOKUPS_PER_S / 1e9, 1),
