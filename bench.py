@@ -130,22 +130,39 @@ def main():
     measured_peak = ops.lds_gather_peak()
     peak = max(NOMINAL_LDS_LOOKUPS_PER_S, measured_peak)
     hbm_bytes = 4 * (x.size + y.numel()) + 4 * f.size + 131072
-    roofline = {
-        "bound": "lds",
-        "kernel": main_kernel,
-        "achieved": round(achieved / 1e9, 1),
-        "peak": round(peak / 1e9, 1),
-        "unit": "Glookup/s",
-        "frac": round(achieved / peak, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-        "kernel_ms": round(main_ms, 4),
-        "lookups_per_launch": lookups,
-        "peak_nominal": round(NOMINAL_LDS_LOOKUPS_PER_S / 1e9, 1),
-        "peak_measured_ds_read_u16": round(measured_peak / 1e9, 1),
-        "hbm_algorithmic_bytes": hbm_bytes,
-        "hbm_gbps_whole_op": round(hbm_bytes / (ms_per_step * 1e-3) / 1e9, 1),
-        "hbm_frac_whole_op": round(hbm_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-    }
+    if depthwise:
+        # K = kh*kw is too small for LDS reuse: 8 bytes of HBM per output element against 9 lookups, HBM-bound
+        dw_bytes = 4 * (x.size + y.numel()) + f.size * 4 + 131072
+        roofline = {
+            "bound": "hbm",
+            "kernel": main_kernel,
+            "achieved": round(dw_bytes / (main_ms * 1e-3) / 1e9, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(dw_bytes / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel_ms": round(main_ms, 4),
+            "algorithmic_bytes_per_launch": dw_bytes,
+            "lookups_per_launch": lookups,
+            "glookups_per_s": round(achieved / 1e9, 1),
+        }
+    else:
+        roofline = {
+            "bound": "lds",
+            "kernel": main_kernel,
+            "achieved": round(achieved / 1e9, 1),
+            "peak": round(peak / 1e9, 1),
+            "unit": "Glookup/s",
+            "frac": round(achieved / peak, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel_ms": round(main_ms, 4),
+            "lookups_per_launch": lookups,
+            "peak_nominal": round(NOMINAL_LDS_LOOKUPS_PER_S / 1e9, 1),
+            "peak_measured_ds_read_u16": round(measured_peak / 1e9, 1),
+            "hbm_algorithmic_bytes": hbm_bytes,
+            "hbm_gbps_whole_op": round(hbm_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "hbm_frac_whole_op": round(hbm_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        }
 
     cpu = None
     if not args.no_cpu_baseline and not depthwise:

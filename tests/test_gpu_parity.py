@@ -210,6 +210,10 @@ DEPTHWISE = [
     ((1, 8, 8, 3), (5, 5, 3, 1), (1, 1), "VALID"),
     ((2, 28, 28, 192), (3, 3, 192, 1), (1, 1), "SAME"),   # MobileNetV2-style block at reduced size
     ((2, 28, 28, 192), (3, 3, 192, 1), (2, 2), "SAME"),
+    ((1, 9, 75, 5), (3, 3, 5, 1), (1, 1), "SAME"),        # rows longer than one sliding-window run
+    ((1, 9, 75, 5), (3, 3, 5, 1), (1, 2), "VALID"),
+    ((1, 20, 20, 6), (3, 3, 6, 1), (3, 3), "SAME"),       # stride outside the sliding-window kernel
+    ((1, 12, 12, 4), (3, 2, 4, 1), (1, 1), "SAME"),
 ]
 
 

@@ -62,21 +62,176 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut_kernel(const Dept
     }
 }
 
+// 3x3 filters, dilation 1, column stride SW in {1, 2}: a thread owns one channel of a run of consecutive output
+// pixels of one output row and slides the 3x3 window along it.  Every input value is loaded and quantized once
+// per window row instead of once per tap, the nine filter codes of the channel live in registers as table row
+// offsets, and no 64-bit index arithmetic is left in the loop.  Same results as depthwise_lut_kernel: taps in
+// (kh, kw) order, zeros (code = zero point) outside the image.
+template <int SW, bool OUT_I32>
+__global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const DepthwiseParams p, const int seg_len,
+                                                                          const int nseg)
+{
+    const int tid = threadIdx.x;
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(p.tableT);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds_dw);
+#pragma unroll
+        for (int i = 0; i < kTableBytes / 16 / kBlockThreads; ++i)
+            dst[tid + i * kBlockThreads] = src[tid + i * kBlockThreads];
+    }
+    __syncthreads();
+
+    const uint32_t zero_off = quantize_code(0.0f, p.in_offset, p.in_inv_scale) * 2u;
+    const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;   // (output row segment, channel), channel fastest
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t item = (int64_t)blockIdx.x * blockDim.x + tid; item < items; item += stride) {
+        const int c = (int)(item % p.C);
+        const int64_t rs = item / p.C;
+        const int seg = (int)(rs % nseg);
+        const int64_t row = rs / nseg;                         // n * OH + oh
+        const int oh = (int)(row % p.OH);
+        const int n = (int)(row / p.OH);
+        const int ow0 = seg * seg_len;
+        const int ow1 = ow0 + seg_len < p.OW ? ow0 + seg_len : p.OW;
+        const int ih0 = oh * p.sh - p.ph;
+
+        uint32_t wrow[9];                                      // byte offset of the table row of each tap's filter code
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+            wrow[t] = (uint32_t)p.wcodes[t * p.C + c] * 512u;
+        const float fs = OUT_I32 ? 0.0f : p.fsum[c];
+        const float *rowp[3];
+        bool rowok[3];
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh) {
+            const int ih = ih0 + kh;
+            rowok[kh] = (unsigned)ih < (unsigned)p.H;
+            rowp[kh] = p.x + ((int64_t)n * p.H + (rowok[kh] ? ih : 0)) * p.W * p.C + c;
+        }
+        float val[3][3];
+        uint32_t off[3][3];                                    // activation code * 2 = byte offset inside a table row
+        auto fetch = [&](int kh, int iw, float &v, uint32_t &o) {
+            v = 0.0f;
+            o = zero_off;
+            if (rowok[kh] && (unsigned)iw < (unsigned)p.W) {
+                v = rowp[kh][iw * p.C];
+                o = quantize_code(v, p.in_offset, p.in_inv_scale) * 2u;
+            }
+        };
+        const int iw0 = ow0 * SW - p.pw;                       // input column under tap kw = 0 of the first output
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw)
+                fetch(kh, iw0 + kw, val[kh][kw], off[kh][kw]);
+        // The columns that enter the window for the next U outputs are loaded one group ahead, so that a thread
+        // keeps 3 * U * SW loads in flight instead of waiting for each output's own.
+        constexpr int U = 4, NC = U * SW;
+        const int len = ow1 - ow0;
+        float pf[3][NC];
+        auto prefetch = [&](int jfirst) {                       // new columns of outputs jfirst .. jfirst + U - 1
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+                for (int t = 0; t < NC; ++t) {
+                    const int j = jfirst + t / SW;               // the output this column first serves
+                    const int iw = iw0 + jfirst * SW + (3 - SW) + t;
+                    pf[kh][t] = 0.0f;
+                    if (j < len && rowok[kh] && (unsigned)iw < (unsigned)p.W)
+                        pf[kh][t] = rowp[kh][iw * p.C];
+                }
+        };
+        prefetch(1);
+        int64_t o_idx = ((int64_t)row * p.OW + ow0) * p.C + c;
+        for (int j0 = 0; j0 < len; j0 += U) {
+            float cur[3][NC];
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+                for (int t = 0; t < NC; ++t)
+                    cur[kh][t] = pf[kh][t];
+            if (j0 + U + 1 < len + U)                            // something left to fetch for the next group
+                prefetch(j0 + U + 1);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (j0 + u >= len)
+                    break;
+                int32_t acc = 0;
+                float psum = 0.0f;
+#pragma unroll
+                for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+                    for (int kw = 0; kw < 3; ++kw) {
+                        psum = __fadd_rn(psum, val[kh][kw]);
+                        acc += (int32_t)*reinterpret_cast<const uint16_t *>(lds_dw + wrow[kh * 3 + kw] + off[kh][kw]);
+                    }
+                if (OUT_I32) {
+                    p.out_i[o_idx] = acc;
+                } else {
+                    const float t0 = __fmul_rn((float)acc, p.s1xs2);
+                    const float t1 = __fmul_rn(p.m2, psum);
+                    const float t2 = __fadd_rn(t0, t1);
+                    const float t3 = __fmul_rn(p.m1, fs);
+                    const float t4 = __fadd_rn(t2, t3);
+                    p.out_f[o_idx] = __fsub_rn(t4, p.k_m1xm2);
+                }
+                o_idx += p.C;
+                // slide the window to output j0 + u + 1: its new columns are cur[.][u*SW .. u*SW + SW - 1]
+                const int iw_new = iw0 + (j0 + u + 1) * SW + (3 - SW);
+#pragma unroll
+                for (int kh = 0; kh < 3; ++kh) {
+#pragma unroll
+                    for (int kw = 0; kw + SW < 3; ++kw) {
+                        val[kh][kw] = val[kh][kw + SW];
+                        off[kh][kw] = off[kh][kw + SW];
+                    }
+#pragma unroll
+                    for (int t = 0; t < SW; ++t) {
+                        const int kw = 3 - SW + t;
+                        const float v = cur[kh][u * SW + t];
+                        const bool inb = rowok[kh] && (unsigned)(iw_new + t) < (unsigned)p.W;
+                        val[kh][kw] = v;
+                        off[kh][kw] = inb ? quantize_code(v, p.in_offset, p.in_inv_scale) * 2u : zero_off;
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename Kernel, typename... Args>
+static hipError_t launch_with_table_lds(Kernel kernel, int grid, hipStream_t stream, Args... args)
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kTableBytes);
+    if (e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBlockThreads), kTableBytes, stream, args...);
+    return hipGetLastError();
+}
+
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream)
 {
-    hipError_t e;
-    if (out_i32) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_lut_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kTableBytes);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(depthwise_lut_kernel<true>, dim3(grid), dim3(kBlockThreads), kTableBytes, stream, p);
-    } else {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_lut_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kTableBytes);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(depthwise_lut_kernel<false>, dim3(grid), dim3(kBlockThreads), kTableBytes, stream, p);
+    const bool sliding = p.KH == 3 && p.KW == 3 && p.dh == 1 && p.dw == 1 && (p.sw == 1 || p.sw == 2) &&
+                         (int64_t)p.W * p.C < (1ll << 31) / 4;
+    if (sliding) {
+        // runs of at most 32 output pixels per thread: enough items to balance the CUs, few window restarts
+        const int nseg = (p.OW + 31) / 32;
+        const int seg_len = (p.OW + nseg - 1) / nseg;
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess)
+            (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;
+        const int64_t blocks = (items + kBlockThreads - 1) / kBlockThreads;
+        const int g3 = (int)(blocks < cus ? blocks : cus);
+        if (p.sw == 1)
+            return out_i32 ? launch_with_table_lds(depthwise_lut3x3_kernel<1, true>, g3, stream, p, seg_len, nseg)
+                           : launch_with_table_lds(depthwise_lut3x3_kernel<1, false>, g3, stream, p, seg_len, nseg);
+        return out_i32 ? launch_with_table_lds(depthwise_lut3x3_kernel<2, true>, g3, stream, p, seg_len, nseg)
+                       : launch_with_table_lds(depthwise_lut3x3_kernel<2, false>, g3, stream, p, seg_len, nseg);
     }
-    return hipGetLastError();
+    return out_i32 ? launch_with_table_lds(depthwise_lut_kernel<true>, grid, stream, p)
+                   : launch_with_table_lds(depthwise_lut_kernel<false>, grid, stream, p);
 }
 
 // ---- LDS gather-rate probe: conflict-free ds_read_u16, 16 wavefronts per CU ------------------
