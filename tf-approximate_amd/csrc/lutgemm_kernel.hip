@@ -346,6 +346,58 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         }
 
         // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----
+        // A lane holds NT consecutive columns of its pixel: stored as they are, one instruction would touch 64
+        // different 64-byte pieces of memory.  The wavefront therefore turns each of its wavefront-rows
+        // through a private piece of LDS (every buffer is free after the last phase) so that NT/4 neighbouring
+        // lanes write one pixel's NT columns: 16 or 8 contiguous runs per store instruction.
+        constexpr bool kTransposed = NT <= 32;
+        if (kTransposed && (g.Co & 3) == 0) {
+            constexpr int Q = NT / 4;                 // 16-byte quads (lanes) per pixel
+            constexpr int PITCH = NT * 4 + 16;        // bytes per pixel in LDS: the +16 spreads pixels over the banks
+            unsigned char *const wl = lds + (size_t)wave * 64 * PITCH;
+            typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r >= (int)nr_s)
+                    break;
+                const int64_t m0 = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
+                const int nvalid = (int)(row_end - m0 < 64 ? row_end - m0 : 64);
+                const float psum = (!OUT_I32 && lane < nvalid) ? p.psum[m0 + lane] : 0.0f;
+                const float t1 = __fmul_rn(p.m2, psum);
+#pragma unroll
+                for (int set = 0; set < SETS; ++set) {
+                    const int h = (c0 + set) & (SETS - 1);
+                    uint32_t w[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (OUT_I32) {
+                            w[e] = (uint32_t)acc[r][set * 8 + e];
+                        } else {
+                            int col = ct * NT + h * 8 + e;
+                            col = col < g.Co ? col : g.Co - 1;
+                            const float t0 = __fmul_rn((float)acc[r][set * 8 + e], p.s1xs2);
+                            const float t2 = __fadd_rn(t0, t1);
+                            const float t3 = __fmul_rn(p.m1, p.fsum[col]);
+                            const float t4 = __fadd_rn(t2, t3);
+                            w[e] = __float_as_uint(__fsub_rn(t4, p.k_m1xm2));
+                        }
+                    }
+                    u32x4s lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
+                    *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32) = lo;
+                    *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32 + 16) = hi;
+                }
+                const int quad = lane % Q, col = ct * NT + quad * 4;
+                uint32_t *const out = OUT_I32 ? reinterpret_cast<uint32_t *>(p.out_i) : reinterpret_cast<uint32_t *>(p.out_f);
+#pragma unroll
+                for (int i = 0; i < Q; ++i) {
+                    const int pix = i * (64 / Q) + lane / Q;
+                    const u32x4s d = *reinterpret_cast<const u32x4s *>(wl + pix * PITCH + quad * 16);
+                    if (pix < nvalid && col < g.Co)
+                        *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + col) = d;
+                }
+            }
+            continue;
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (!rvalid[r])
