@@ -54,6 +54,10 @@ def main():
     ap.add_argument("--codes", default="uniform", choices=["uniform", "halfnormal"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--network", default=None,
+                    help="instead of the single layer, time a whole synthetic network whose convolutions all run "
+                         "through the op (tf-approximate_amd/networks.py: cifar_resnet_b128, resnet50_b64, "
+                         "inverted_residual_b64_s1, inverted_residual_b64_s2) and report images/s")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run a plain device copy of MIB MiB five times: the known-size "
                          "kernel that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -76,6 +80,28 @@ def main():
     import __graft_entry__ as entry
     pkg = entry.load_package()
     from tf_approximate_amd import ops, synth
+
+    if args.network:
+        from tf_approximate_amd import networks
+        table = synth.table_uniform_error(11) if args.network.startswith("resnet50") else synth.table_noisy(7)
+        net, xin = networks.build(args.network, table)
+        _, macs = net.forward(xin, calibrate=True)          # fixes every layer's min/max from its own tensors
+        for _ in range(max(args.warmup, 1)):
+            net.forward(xin)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            net.forward(xin)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        print(json.dumps({
+            "metric": "images_per_s", "value": round(xin.shape[0] / (ms * 1e-3), 1), "unit": "images/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "int32", "data": "synthetic",
+            "config": {"workload": args.network, "input": list(xin.shape), "convolutions": net.conv_count(),
+                       "approx_macs_per_pass": macs, "note": "convolutions through the op; ReLU, adds, max-pool in torch"},
+            "approx_gmac_per_s": round(macs / (ms * 1e-3) / 1e9, 1)}))
+        return
 
     xs, fs, strides, depthwise = WORKLOADS[args.workload]
     mm = (-1.0, 1.0, -0.5, 0.5)

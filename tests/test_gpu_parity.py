@@ -283,3 +283,28 @@ def test_non_default_stream(pkg, oracle):
     s.synchronize()
     rc, y_ref, _ = oracle.conv2d_fast(table, case["x"], case["f"], *case["minmax"], threads=8)
     assert refimpl.linf_rel(y.cpu().numpy(), y_ref) <= TOL
+
+
+@pytest.mark.parametrize("name", ["cifar", "inverted_residual_s2"])
+def test_network_layers_vs_oracle(pkg, oracle, name):
+    """Every convolution of a small synthetic network, checked on the tensors the network itself produced."""
+    import torch
+    from tf_approximate_amd import networks
+    table = pkg.synth.table_noisy(7)
+    if name == "cifar":
+        prog, shape = networks.cifar_resnet_program(blocks_per_stage=1), (2, 16, 16, 3)
+    else:
+        prog, shape = networks.inverted_residual_program(8, 6, 2), (2, 14, 14, 8)
+    net = networks.ApproxNetwork(prog, shape, table, seed=3)
+    x = torch.from_numpy(np.random.default_rng(5).uniform(0, 1, size=shape).astype(np.float32)).to(net.device)
+    trace = []
+    net.forward(x, calibrate=True, trace=trace)
+    assert len(trace) == net.conv_count()
+    for spec, xin, w, mm, y in trace:
+        strides = (spec.stride, spec.stride)
+        if spec.depthwise:
+            rc, y_ref, _ = oracle.depthwise_conv2d(table, xin, w, *mm, strides=strides, padding="SAME", dilations=(1, 1))
+        else:
+            rc, y_ref, _ = oracle.conv2d_fast(table, xin, w, *mm, strides=strides, padding="SAME", dilations=(1, 1))
+        assert rc == 0
+        assert refimpl.linf_rel(y, y_ref) <= 1e-5
