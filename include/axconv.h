@@ -95,6 +95,11 @@ int axc_conv2d_geometry(const axc_conv2d_desc *desc, axc_conv2d_dims *dims);
 /* Scratch the launch calls below need for this desc (replaces the three allocate_temp calls at
  * approx_nn_conv_ops.cpp:590-613). */
 int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
+
+/* How the dense kernel would cut this layer on the current device (for tools and tests; the reference has no
+ * counterpart, its launch shapes are fixed in cuda/approx_nn_conv_kernels.cu:296-627):
+ * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups }. */
+int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6]);
 int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
 
 /* The op: replaces ApproxConv2DOp::Compute -> LaunchApproxConv2DOp<GPUDevice> and the kernels it

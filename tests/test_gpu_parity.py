@@ -125,6 +125,9 @@ MEDIUM = [
     ((2, 56, 56, 64), (3, 3, 64, 64), (1, 1)),      # north-star layer at batch 2
     ((1, 28, 28, 128), (1, 1, 128, 256), (1, 1)),   # 1x1 expand
     ((1, 30, 30, 24), (7, 7, 24, 64), (2, 2)),      # 7x7/2 stem shape
+    ((2, 7, 7, 512), (3, 3, 512, 64), (1, 1)),      # few pixels, long K: the tile plan splits K over tiles
+    ((4, 7, 7, 256), (1, 1, 256, 30), (1, 1)),      # split K with a column count that is no multiple of 4
+    ((2, 14, 14, 96), (3, 3, 96, 48), (1, 1)),
 ]
 
 
@@ -308,3 +311,11 @@ def test_network_layers_vs_oracle(pkg, oracle, name):
             rc, y_ref, _ = oracle.conv2d_fast(table, xin, w, *mm, strides=strides, padding="SAME", dilations=(1, 1))
         assert rc == 0
         assert refimpl.linf_rel(y, y_ref) <= 1e-5
+
+
+def test_split_k_plan_is_exercised(pkg):
+    """The cases above named for it really run with K split over tiles (and the north-star layer does not)."""
+    from tf_approximate_amd import ops
+    assert ops.conv2d_tile_plan((2, 7, 7, 512), (3, 3, 512, 64))["k_splits"] > 1
+    assert ops.conv2d_tile_plan((4, 7, 7, 256), (1, 1, 256, 30))["k_splits"] > 1
+    assert ops.conv2d_tile_plan((64, 56, 56, 64), (3, 3, 64, 64))["k_splits"] == 1

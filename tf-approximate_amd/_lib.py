@@ -54,6 +54,7 @@ SYMBOLS = [
     ("axc_quant_props_compute", ctypes.c_int, [_f, _f, _f, _f, ctypes.POINTER(QuantProps)]),
     ("axc_conv2d_geometry", ctypes.c_int, [_desc, ctypes.POINTER(ConvDims)]),
     ("axc_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
+    ("axc_conv2d_tile_plan", ctypes.c_int, [_desc, ctypes.POINTER(ctypes.c_int32)]),
     ("axc_depthwise_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),

@@ -303,19 +303,32 @@ DensePlan make_plan(const ConvGeom &g, int cus)
             cands.push_back(total_wrows);
         for (int64_t n_row : cands) {
             const int64_t wrows = (total_wrows + n_row - 1) / n_row;  // per tile
-            const int64_t tiles = n_row * n_col;
-            const int64_t rounds = (tiles + cus - 1) / cus;
             const double per_simd = (double)((wrows + 3) / 4);          // wavefront-rows on the busiest SIMD
-            const double per_fill = 450.0 + per_simd * (64.0 * 1.3 * 4.0); // cycles: derive + lookups
-            const double cost = (double)rounds * ((double)fills * per_fill + 3000.0);
-            if (cost < best_cost) {
-                best_cost = cost;
-                best.nt = nt;
-                best.rows_per_tile = (int)(wrows * 64);
-                best.n_row_tiles = (int)((total_wrows + wrows - 1) / wrows);
-                best.n_col_tiles = n_col;
-                best.fills = fills;
-                best.grid = (int)((int64_t)best.n_row_tiles * n_col < cus ? (int64_t)best.n_row_tiles * n_col : cus);
+            // cycles per fill, fitted to measurements: barrier + expanding + staging, then the lookups
+            const double per_fill = 1700.0 + per_simd * 290.0;
+            // Splitting K over tiles keeps the tiles tall (many lookups per expanded fill) when M alone does not
+            // give every CU a tile; the int32 partial sums then cost one more pass over (k_splits + 1) outputs.
+            for (int ks : {1, 2, 3, 4, 6, 8, 12, 16}) {
+                const int fps = (fills + ks - 1) / ks;
+                if (ks > 1 && (fps < 8 || (int64_t)(ks - 1) * fps >= fills))
+                    continue;
+                const int64_t tiles = n_row * n_col * ks;
+                const int64_t rounds = (tiles + cus - 1) / cus;
+                double cost = (double)rounds * ((double)fps * per_fill + 6000.0);
+                if (ks > 1) // the extra pass, and a margin: split only for a clear gain
+                    cost = cost * 1.08 + 20000.0 + (double)(ks + 1) * (double)g.M * g.Co * 4.0 * 7e-4;
+                if (cost < best_cost) {
+                    best_cost = cost;
+                    best.nt = nt;
+                    best.rows_per_tile = (int)(wrows * 64);
+                    best.n_row_tiles = (int)((total_wrows + wrows - 1) / wrows);
+                    best.n_col_tiles = n_col;
+                    best.fills = fills;
+                    best.k_splits = ks;
+                    best.fills_per_split = fps;
+                    const int64_t all = (int64_t)best.n_row_tiles * n_col * ks;
+                    best.grid = (int)(all < cus ? all : cus);
+                }
             }
         }
     }
@@ -325,7 +338,7 @@ DensePlan make_plan(const ConvGeom &g, int cus)
 inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct DenseWorkspace {
-    size_t xq_off, psum_off, wq_off, fsum_off, total;
+    size_t xq_off, psum_off, wq_off, fsum_off, part_off, total;
 };
 
 DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
@@ -336,6 +349,9 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
     w.psum_off = off; off += align_up((size_t)g.M * 4); // patch sums: one float per output pixel
     w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
     w.fsum_off = off; off += align_up((size_t)g.Co * 4);
+    w.part_off = off;   // int32 partial sums of the K splits
+    if (plan.k_splits > 1)
+        off += align_up((size_t)plan.k_splits * (size_t)g.M * g.Co * 4);
     w.total = off;
     return w;
 }
@@ -401,11 +417,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
 
     if (g.K == 0) { // no taps: every sum is empty
         const int64_t n = g.M * g.Co;
-        if (out_i) {
-            AXC_HIP(hipMemsetAsync(out_i, 0, (size_t)n * 4, stream));
-        } else {
-            AXC_HIP(hipMemsetAsync(out_f, 0, (size_t)n * 4, stream));
-        }
+        // a fill kernel rather than hipMemsetAsync: callers may capture the stream into a graph
+        AXC_HIP(launch_fill_u32(out_i ? reinterpret_cast<uint32_t *>(out_i) : reinterpret_cast<uint32_t *>(out_f), n, 0u,
+                                stream));
         return AXC_OK;
     }
     if (workspace_bytes < pd.ws.total || (!workspace && pd.ws.total))
@@ -457,6 +471,18 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     p.zp4 = zp4;
     p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
     p.wq_bytes = (uint32_t)((size_t)pd.plan.n_col_tiles * pd.plan.fills * 128);
+    if (pd.plan.k_splits > 1) {
+        int32_t *part = reinterpret_cast<int32_t *>(ws + pd.ws.part_off);
+        p.out_f = nullptr;
+        p.out_i = part;
+        {
+            ProfScope ps("lutgemm_expand", stream);
+            AXC_HIP(launch_dense(p, true, stream));
+        }
+        ProfScope ps("splitk_epilogue", stream);
+        AXC_HIP(launch_splitk_epilogue(p, part, out_f, out_i, stream));
+        return AXC_OK;
+    }
     {
         ProfScope ps("lutgemm_expand", stream);
         AXC_HIP(launch_dense(p, out_i != nullptr, stream));
@@ -635,6 +661,23 @@ int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes)
     if (rc != AXC_OK)
         return rc;
     *bytes = pd.ws.total;
+    return AXC_OK;
+}
+
+int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6])
+{
+    if (!plan)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    PreparedDense pd;
+    int rc = prepare_dense(desc, &pd);
+    if (rc != AXC_OK)
+        return rc;
+    plan[0] = pd.plan.nt;
+    plan[1] = pd.plan.rows_per_tile;
+    plan[2] = pd.plan.n_row_tiles;
+    plan[3] = pd.plan.n_col_tiles;
+    plan[4] = pd.plan.k_splits;
+    plan[5] = pd.plan.grid;
     return AXC_OK;
 }
 

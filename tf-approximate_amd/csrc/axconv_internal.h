@@ -37,7 +37,9 @@ struct DensePlan {
     int nt;                // columns per tile: 16, 32 or 64
     int rows_per_tile;     // multiple of 64, <= 1024 * (64 / nt)
     int n_row_tiles, n_col_tiles;
-    int fills;             // expanded-row refills per tile: KH*KW * C4 * (4 / (64/nt))
+    int fills;             // expanded-row refills over the whole K: KH*KW * C4 * (4 / (64/nt))
+    int k_splits;          // tiles along K: each computes fills_per_split fills into its own int32 partial sums
+    int fills_per_split;
     int grid;
 };
 
@@ -51,7 +53,7 @@ struct DenseParams {
     const float *fsum;      // [Co] sum over (h, w, c) of the raw filter
     const uint16_t *tableT; // [257 filter code (256 = null)][256 input code]
     float *out_f;
-    int32_t *out_i;
+    int32_t *out_i;         // with k_splits > 1: [k_splits][M][Co] partial sums, reduced by launch_splitk_epilogue
     float s1xs2, m1, m2, k_m1xm2; // epilogue constants; k_m1xm2 = float(K) * m1xM2
     uint32_t zp4;           // row-permuted zero code replicated in all four bytes
     uint32_t xq_bytes, wq_bytes; // sizes of the two streams (buffer-descriptor bounds)
@@ -96,6 +98,9 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
 hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
                                 hipStream_t stream);
 hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream);
+hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials, float *out_f, int32_t *out_i,
+                                  hipStream_t stream);
+hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t stream);
 hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
                                    uint8_t *wcodes, float *fsum, hipStream_t stream);
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream);

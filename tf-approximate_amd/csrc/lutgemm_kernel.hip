@@ -137,8 +137,10 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     unsigned char *const stage = lds + 2 * kExpandBytes;
 
     const int taps = g.KH * g.KW;
-    const int ntiles = p.plan.n_row_tiles * p.plan.n_col_tiles;
-    const int fills = p.plan.fills;
+    // a tile = (row tile, column tile, K split); the K splits of a column tile count as further column tiles
+    const int nct_v = p.plan.n_col_tiles * p.plan.k_splits;
+    const int ntiles = p.plan.n_row_tiles * nct_v;
+    const int fills_all = p.plan.fills;
     const int rowstep = g.C4 * g.W; // dwords between input rows in xq
     // xq ends with one extra input row filled with the zero-point code: taps outside the image read it
     const uint32_t zp_row = p.xq_bytes;
@@ -153,7 +155,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         // inside a group of 8 * n_col_tiles consecutive tiles, tile r is (row tile r % 8, column tile r / 8).
         int ct, rt;
         {
-            const int nct = p.plan.n_col_tiles, group = 8 * nct;
+            const int nct = nct_v, group = 8 * nct;
             const int gi = tile / group, r = tile - gi * group;
             if ((gi + 1) * group <= ntiles) {
                 ct = r >> 3;
@@ -163,6 +165,10 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 rt = tile / nct;
             }
         }
+        const int ksi = ct / p.plan.n_col_tiles;           // K split of this tile
+        ct -= ksi * p.plan.n_col_tiles;
+        const int f0 = ksi * p.plan.fills_per_split;        // its fills: [f0, f0 + fills)
+        const int fills = fills_all - f0 < p.plan.fills_per_split ? fills_all - f0 : p.plan.fills_per_split;
         const int64_t row0 = (int64_t)rt * p.plan.rows_per_tile;
         const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
 
@@ -205,10 +211,12 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             for (int j = 0; j < NT; ++j)
                 acc[r][j] = 0;
 
-        const uint32_t wq_tile = (uint32_t)ct * (uint32_t)fills * 128u; // byte offset of this tile's codes
+        const uint32_t wq_tile = ((uint32_t)ct * (uint32_t)fills_all + (uint32_t)f0) * 128u; // this tile's first codes
+        const int fills_left = fills_all - f0;              // codes may be prefetched past the split, not past the end
 
         // ---- activation cursor: position (tap, quad) of the fill whose activations are fetched next ----
-        int cur_fill = 0, cur_q = 0, cur_kh = 0, cur_kw = 0, cur_sub = 0;
+        int cur_fill = 0, cur_sub = f0 % SUBS;
+        int cur_q = (f0 / SUBS) % g.C4, cur_kh = (f0 / SUBS / g.C4) / g.KW, cur_kw = (f0 / SUBS / g.C4) % g.KW;
         uint32_t idx_tap[R];   // byte offset in xq of quad 0 of the current tap (the zero-point row outside)
         auto tap_setup = [&]() {
             const int dh = cur_kh * g.dh, dw = cur_kw * g.dw;
@@ -236,7 +244,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 if (++cur_q == g.C4) {
                     cur_q = 0;
                     if (++cur_kw == g.KW) { cur_kw = 0; ++cur_kh; }
-                    if (cur_fill < fills)
+                    if (cur_fill < fills_left)
                         tap_setup();
                 }
             }
@@ -244,7 +252,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
 
         // ---- table rows of one fill: global -> registers -> staged rows -> expanded rows ----
         auto load_codes = [&](int fill, uint32_t (&codes)[4]) {
-            const uint32_t f = (uint32_t)(fill < fills ? fill : fills - 1);
+            const uint32_t f = (uint32_t)(fill < fills_left ? fill : fills_left - 1);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 codes[j] = __builtin_amdgcn_raw_buffer_load_b16(wq_rsrc, (int)((st_slot + 16u * j) * 2u),
@@ -323,12 +331,12 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         const uint32_t nr_s = __builtin_amdgcn_readfirstlane(nr);
         // Entering phase p the activation cursor stands on fill p+1 and shift_cur belongs to fill p; the cursor
         // is moved on behind the phase body, where most wavefronts would otherwise only wait for the barrier.
-        uint32_t shift_cur = 0;
+        uint32_t shift_cur = (uint32_t)cur_sub * (32u / SUBS);
         if (fills > 1)
             advance_cursor();
         auto phase = [&](const int pcur, uint32_t (&act_cur)[R], uint32_t (&act_next)[R], auto buf_tag) {
             constexpr int BUF = decltype(buf_tag)::value;
-            const int fcodes = pcur + 4 < fills ? pcur + 4 : fills - 1;
+            const int fcodes = pcur + 4 < fills_left ? pcur + 4 : fills_left - 1;
             const uint32_t cso = wq_tile + (uint32_t)fcodes * 128u;
             const uint32_t qoff = (uint32_t)(cur_q * g.W * 4);
             phase_body<NT, BUF>(acc, act_cur, act_next, idx_tap, rows, codes, k, nr_s,
@@ -387,7 +395,8 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                     *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32 + 16) = hi;
                 }
                 const int quad = lane % Q, col = ct * NT + quad * 4;
-                uint32_t *const out = OUT_I32 ? reinterpret_cast<uint32_t *>(p.out_i) : reinterpret_cast<uint32_t *>(p.out_f);
+                uint32_t *const out = OUT_I32 ? reinterpret_cast<uint32_t *>(p.out_i) + (int64_t)ksi * g.M * g.Co
+                                              : reinterpret_cast<uint32_t *>(p.out_f);
 #pragma unroll
                 for (int i = 0; i < Q; ++i) {
                     const int pix = i * (64 / Q) + lane / Q;
@@ -419,13 +428,13 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                         typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
                         i32x4 lo = {acc[r][set * 8 + 0], acc[r][set * 8 + 1], acc[r][set * 8 + 2], acc[r][set * 8 + 3]};
                         i32x4 hi = {acc[r][set * 8 + 4], acc[r][set * 8 + 5], acc[r][set * 8 + 6], acc[r][set * 8 + 7]};
-                        *reinterpret_cast<i32x4 *>(p.out_i + o) = lo;
-                        *reinterpret_cast<i32x4 *>(p.out_i + o + 4) = hi;
+                        *reinterpret_cast<i32x4 *>(p.out_i + (int64_t)ksi * g.M * g.Co + o) = lo;
+                        *reinterpret_cast<i32x4 *>(p.out_i + (int64_t)ksi * g.M * g.Co + o + 4) = hi;
                     } else {
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
                             if (col0 + e < g.Co)
-                                p.out_i[o + e] = acc[r][set * 8 + e];
+                                p.out_i[(int64_t)ksi * g.M * g.Co + o + e] = acc[r][set * 8 + e];
                     }
                 } else {
                     float v[8];

@@ -400,6 +400,76 @@ __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t *__restrict__ ds
         dst[i] = value;
 }
 
+hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t stream)
+{
+    for (int64_t done = 0; done < n; done += (int64_t)1 << 30) { // int-sized pieces
+        const int piece = (int)(n - done < ((int64_t)1 << 30) ? n - done : (int64_t)1 << 30);
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks_for(piece, 256)), dim3(256), 0, stream, dst + done, piece, value);
+    }
+    return hipGetLastError();
+}
+
+// Reduction of the K splits' int32 partial sums (exact, so the order does not matter) followed by the op's
+// epilogue (approx_nn_conv_kernels.cpp:250-253), four consecutive columns per thread when Co % 4 == 0.
+template <int V>
+__global__ void __launch_bounds__(256) splitk_epilogue_kernel(const int32_t *__restrict__ part, int ks, int64_t mc,
+                                                               int Co, const float *__restrict__ psum,
+                                                               const float *__restrict__ fsum, float s1xs2, float m1,
+                                                               float m2, float k_m1xm2, float *__restrict__ out_f,
+                                                               int32_t *__restrict__ out_i)
+{
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+    if (i >= mc)
+        return;
+    int32_t a[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+        a[e] = 0;
+    for (int k = 0; k < ks; ++k) {
+        if (V == 4) {
+            const int4 v = *reinterpret_cast<const int4 *>(part + (int64_t)k * mc + i);
+            a[0] += v.x; a[1 % V] += v.y; a[2 % V] += v.z; a[3 % V] += v.w;
+        } else {
+            a[0] += part[(int64_t)k * mc + i];
+        }
+    }
+    if (out_i) {
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+            out_i[i + e] = a[e];
+        return;
+    }
+    const int64_t m = i / Co;
+    const int col = (int)(i - m * Co);
+    const float t1 = __fmul_rn(m2, psum[m]);
+    float r[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        const float t0 = __fmul_rn((float)a[e], s1xs2);
+        const float t2 = __fadd_rn(t0, t1);
+        const float t3 = __fmul_rn(m1, fsum[col + e]);
+        const float t4 = __fadd_rn(t2, t3);
+        r[e] = __fsub_rn(t4, k_m1xm2);
+    }
+    if (V == 4)
+        *reinterpret_cast<float4 *>(out_f + i) = make_float4(r[0], r[1 % V], r[2 % V], r[3 % V]);
+    else
+        out_f[i] = r[0];
+}
+
+hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials, float *out_f, int32_t *out_i,
+                                  hipStream_t stream)
+{
+    const int64_t mc = p.g.M * p.g.Co;
+    if ((p.g.Co & 3) == 0)
+        hipLaunchKernelGGL(splitk_epilogue_kernel<4>, dim3(blocks_for(mc / 4, 256)), dim3(256), 0, stream, partials,
+                           p.plan.k_splits, mc, p.g.Co, p.psum, p.fsum, p.s1xs2, p.m1, p.m2, p.k_m1xm2, out_f, out_i);
+    else
+        hipLaunchKernelGGL(splitk_epilogue_kernel<1>, dim3(blocks_for(mc, 256)), dim3(256), 0, stream, partials,
+                           p.plan.k_splits, mc, p.g.Co, p.psum, p.fsum, p.s1xs2, p.m1, p.m2, p.k_m1xm2, out_f, out_i);
+    return hipGetLastError();
+}
+
 static hipError_t launch_zero_point_row(const ConvGeom &g, uint32_t zp4, uint32_t *xq, hipStream_t stream)
 {
     const int n = g.C4 * g.W;
