@@ -1,4 +1,4 @@
-"""Full-size layers (BASELINE.json configs 4 and 5): too large for the CPU oracle to recompute whole,
+"""Full-size layers (the ResNet-50-shaped and the large GEMM-dominated benchmark layers): too large for the CPU oracle to recompute whole,
 so checked through size-independent properties and through oracle evaluation of sampled output pixels."""
 import numpy as np
 import pytest
@@ -104,7 +104,7 @@ def test_north_star_layer_is_deterministic(pkg, north_star):
 @pytest.mark.parametrize("name", ["A_1x1_256_1024", "B_3x3_512_512", "stem_7x7", "stage4_3x3"])
 @pytest.mark.parametrize("tname", ["random", "exact"])
 def test_stress_layers_sampled_pixels(pkg, oracle, name, tname):
-    """BASELINE.json config 5 (A: 1x1 32x56x56x256->1024; B: 3x3 64x28x28x512->512, K = 4608) and the
+    """The large GEMM-dominated stress layers (A: 1x1 32x56x56x256->1024; B: 3x3 64x28x28x512->512, K = 4608) and the
     ResNet-50 stem / stage-4 shapes, half-normal activation codes, fully random and exact tables."""
     shapes = {
         "A_1x1_256_1024": ((32, 56, 56, 256), (1, 1, 256, 1024), (1, 1)),
