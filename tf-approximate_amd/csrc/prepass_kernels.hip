@@ -13,9 +13,12 @@ namespace axc {
 __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__restrict__ x, int64_t pixels,
                                                                  int H, int W, int C, int C4, float offset,
                                                                  float inv_scale, uint32_t *__restrict__ xq,
-                                                                 float *__restrict__ chsum)
+                                                                 float *__restrict__ chsum, uint32_t zp4)
 {
     const int64_t pix = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    // the extra [C4][W] row behind the image rows: every dword is the zero-point code x4
+    for (int64_t i = pix; i < (int64_t)C4 * W; i += (int64_t)gridDim.x * blockDim.x)
+        xq[pixels * C4 + i] = zp4;
     if (pix >= pixels)
         return;
     const int w = (int)(pix % W);
@@ -43,9 +46,12 @@ __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__r
 // read consecutive float4 of the NHWC input (one float4 = the four channels of one xq dword).
 __global__ void __launch_bounds__(256) quantize_relayout_vec4_kernel(const float4 *__restrict__ x4, int64_t quads,
                                                                       int W, int C4, float offset, float inv_scale,
-                                                                      uint32_t *__restrict__ xq)
+                                                                      uint32_t *__restrict__ xq, uint32_t zp4)
 {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    // the extra [C4][W] row behind the image rows: every dword is the zero-point code x4
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (int64_t)C4 * W; i += stride)
+        xq[quads + i] = zp4;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) {
         const float4 v = x4[i];
         const int64_t pix = i / C4;
@@ -282,16 +288,14 @@ __global__ void __launch_bounds__(256) codes_relayout_kernel(const uint8_t *__re
 // and pack into the order the LUT-GEMM consumes.
 //   wq[ct][fill][slot], fill = (tap * C4 + q) * SUBS + sub, slot = kk * NT + j
 //   channel = q*4 + sub*KS + kk, column = ct*NT + j; kNullWeight where channel >= C or column >= Co.
-__global__ void __launch_bounds__(256) filter_pack_kernel(const float *__restrict__ filter,
-                                                           const uint8_t *__restrict__ filter_codes, int taps,
-                                                           int C, int C4, int Co, int nt, int n_col_tiles,
-                                                           float offset, float inv_scale,
-                                                           uint16_t *__restrict__ wq)
+__device__ __forceinline__ void filter_pack_element(const int64_t i, const float *__restrict__ filter,
+                                                    const uint8_t *__restrict__ filter_codes, int taps, int C,
+                                                    int C4, int Co, int nt, int n_col_tiles, float offset,
+                                                    float inv_scale, uint16_t *__restrict__ wq)
 {
     const int ks = 64 / nt, subs = 4 / ks;
     const int fills = taps * C4 * subs;
     const int64_t total = (int64_t)n_col_tiles * fills * 64;
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total)
         return;
     const int slot = (int)(i & 63);
@@ -322,13 +326,14 @@ __global__ void __launch_bounds__(256) filter_pack_kernel(const float *__restric
 constexpr int kFsRows = 512, kFsThreads = 1024;
 constexpr int kFsLdsBytes = kFsRows * 65 * 4;
 
-__global__ void __launch_bounds__(kFsThreads) filter_sums_kernel(const float *__restrict__ filter, int K, int Co,
-                                                                  float *__restrict__ fsum)
+extern __shared__ __align__(16) unsigned char fs_lds[];
+
+__device__ __forceinline__ void filter_sums_block(const int block, const float *__restrict__ filter, int K, int Co,
+                                                  float *__restrict__ fsum)
 {
     constexpr int kBatch = 32, kPer = kFsRows * 64 / kFsThreads; // loads per thread per pass
-    extern __shared__ __align__(16) unsigned char fs_lds[];
     float *const stage = reinterpret_cast<float *>(fs_lds);
-    const int col0 = blockIdx.x * 64;
+    const int col0 = block * 64;
     const int t = threadIdx.x;
     const int cl = t & 63, rsub = t >> 6; // 16 rows per step
     float s = 0.0f;
@@ -362,6 +367,23 @@ __global__ void __launch_bounds__(kFsThreads) filter_sums_kernel(const float *__
     }
     if (t < 64 && col0 + t < Co)
         fsum[col0 + t] = s;
+}
+
+// One launch for the whole filter pre-pass: the first sum_blocks workgroups compute the column sums (skipped when
+// fsum is null), the others pack the codes.
+__global__ void __launch_bounds__(kFsThreads) filter_prep_kernel(const float *__restrict__ filter,
+                                                                  const uint8_t *__restrict__ filter_codes, int taps,
+                                                                  int C, int C4, int Co, int nt, int n_col_tiles,
+                                                                  float offset, float inv_scale,
+                                                                  uint16_t *__restrict__ wq, int sum_blocks,
+                                                                  float *__restrict__ fsum)
+{
+    if ((int)blockIdx.x < sum_blocks) {
+        filter_sums_block((int)blockIdx.x, filter, taps * C, Co, fsum);
+        return;
+    }
+    const int64_t i = (int64_t)(blockIdx.x - sum_blocks) * blockDim.x + threadIdx.x;
+    filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, offset, inv_scale, wq);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -481,20 +503,17 @@ static hipError_t launch_zero_point_row(const ConvGeom &g, uint32_t zp4, uint32_
 hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
                                     uint32_t zp4, uint32_t *xq, float *chsum, hipStream_t stream)
 {
-    hipError_t ez = launch_zero_point_row(g, zp4, xq, stream);
-    if (ez != hipSuccess)
-        return ez;
     const int64_t pixels = (int64_t)g.N * g.H * g.W;
     if ((g.C & 3) == 0 && !chsum && ((uintptr_t)x & 15) == 0) {
         const int64_t quads = pixels * g.C4;
         int64_t blocks = (quads + 256 * 4 - 1) / (256 * 4);
         if (blocks > 65536) blocks = 65536;
         hipLaunchKernelGGL(quantize_relayout_vec4_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           reinterpret_cast<const float4 *>(x), quads, g.W, g.C4, offset, inv_scale, xq);
+                           reinterpret_cast<const float4 *>(x), quads, g.W, g.C4, offset, inv_scale, xq, zp4);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(quantize_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, x, pixels,
-                       g.H, g.W, g.C, g.C4, offset, inv_scale, xq, chsum);
+                       g.H, g.W, g.C, g.C4, offset, inv_scale, xq, chsum, zp4);
     return hipGetLastError();
 }
 
@@ -554,18 +573,17 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
                               hipStream_t stream)
 {
     const int64_t total = (int64_t)plan.n_col_tiles * plan.fills * 64;
-    hipLaunchKernelGGL(filter_pack_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, stream, filter,
-                       filter_codes, g.KH * g.KW, g.C, g.C4, g.Co, plan.nt, plan.n_col_tiles, offset, inv_scale,
-                       wq);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess || !fsum || !filter)
-        return e;
-    hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(filter_sums_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kFsLdsBytes);
-    if (ea != hipSuccess)
-        return ea;
-    hipLaunchKernelGGL(filter_sums_kernel, dim3(blocks_for(g.Co, 64)), dim3(kFsThreads), kFsLdsBytes, stream, filter, g.K, g.Co,
-                       fsum);
+    const int sum_blocks = (fsum && filter) ? (int)blocks_for(g.Co, 64) : 0;
+    const size_t lds = sum_blocks ? kFsLdsBytes : 0;
+    if (lds) {
+        hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(filter_prep_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, kFsLdsBytes);
+        if (ea != hipSuccess)
+            return ea;
+    }
+    hipLaunchKernelGGL(filter_prep_kernel, dim3(sum_blocks + blocks_for(total, kFsThreads)), dim3(kFsThreads), lds,
+                       stream, filter, filter_codes, g.KH * g.KW, g.C, g.C4, g.Co, plan.nt, plan.n_col_tiles, offset,
+                       inv_scale, wq, sum_blocks, fsum);
     return hipGetLastError();
 }
 
