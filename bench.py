@@ -58,6 +58,9 @@ def main():
                     help="instead of the single layer, time a whole synthetic network whose convolutions all run "
                          "through the op (tf-approximate_amd/networks.py: cifar_resnet_b128, resnet50_b64, "
                          "inverted_residual_b64_s1, inverted_residual_b64_s2) and report images/s")
+    ap.add_argument("--fused-layers", action="store_true",
+                    help="with --network: every dense convolution through the layer entry point (per-batch min/max "
+                         "and fake quantization on the device, ReLU fused) instead of the op with calibrated ranges")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run a plain device copy of MIB MiB five times: the known-size "
                          "kernel that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -84,7 +87,7 @@ def main():
     if args.network:
         from tf_approximate_amd import networks
         table = synth.table_uniform_error(11) if args.network.startswith("resnet50") else synth.table_noisy(7)
-        net, xin = networks.build(args.network, table)
+        net, xin = networks.build(args.network, table, fused_layers=args.fused_layers)
         _, macs = net.forward(xin, calibrate=True)          # fixes every layer's min/max from its own tensors
         for _ in range(max(args.warmup, 1)):
             net.forward(xin)
@@ -99,7 +102,7 @@ def main():
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "int32", "data": "synthetic",
             "config": {"workload": args.network, "input": list(xin.shape), "convolutions": net.conv_count(),
-                       "approx_macs_per_pass": macs, "note": "convolutions through the op; ReLU, adds, max-pool in torch"},
+                       "approx_macs_per_pass": macs, "fused_layers": bool(args.fused_layers), "note": "convolutions through the op; ReLU, adds, max-pool in torch"},
             "approx_gmac_per_s": round(macs / (ms * 1e-3) / 1e9, 1)}))
         return
 

@@ -96,6 +96,17 @@ int axc_conv2d_geometry(const axc_conv2d_desc *desc, axc_conv2d_dims *dims);
  * approx_nn_conv_ops.cpp:590-613). */
 int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
 
+/* The reference's Keras layer around the op, FakeApproxConv2D.call
+ * (tf2/python/keras/layers/fake_approx_convolutional.py:223-261), as one call that never leaves the device:
+ * min / max of the input batch and of the kernel (reduce_min / reduce_max, :233-241), fake quantization of both
+ * with them (fake_quant_with_min_max_vars, :235,242: here fused into the kernels that read the tensors), the op,
+ * then bias_add and the activation of Conv.call (:261).  bias may be null; activation is AXC_ACT_*.
+ * Workspace: axc_conv2d_workspace_bytes.  Dense convolutions only. */
+enum { AXC_ACT_NONE = 0, AXC_ACT_RELU = 1 };
+int axc_fake_approx_conv2d(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                           const float *filter, const float *bias, int activation, float *output, void *workspace,
+                           size_t workspace_bytes, void *stream);
+
 /* How the dense kernel would cut this layer on the current device (for tools and tests; the reference has no
  * counterpart, its launch shapes are fixed in cuda/approx_nn_conv_kernels.cu:296-627):
  * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups }. */

@@ -319,3 +319,48 @@ def test_split_k_plan_is_exercised(pkg):
     assert ops.conv2d_tile_plan((2, 7, 7, 512), (3, 3, 512, 64))["k_splits"] > 1
     assert ops.conv2d_tile_plan((4, 7, 7, 256), (1, 1, 256, 30))["k_splits"] > 1
     assert ops.conv2d_tile_plan((64, 56, 56, 64), (3, 3, 64, 64))["k_splits"] == 1
+
+
+LAYER_CASES = [
+    # input, filter, strides, bias, activation, input range
+    ((2, 12, 12, 8), (3, 3, 8, 16), (1, 1), True, "relu", (-1.0, 1.0)),
+    ((1, 9, 11, 5), (3, 3, 5, 7), (2, 2), False, None, (0.0, 3.0)),         # zero point 0, odd column count
+    ((2, 7, 7, 256), (3, 3, 256, 32), (1, 1), True, "relu", (-2.0, 0.5)),   # K split over tiles
+    ((1, 16, 16, 3), (1, 1, 3, 4), (1, 1), True, None, (-1.0, 1.0)),
+]
+
+
+@pytest.mark.parametrize("case", LAYER_CASES, ids=[str(i) for i in range(len(LAYER_CASES))])
+def test_fake_approx_conv2d_layer_vs_composition(pkg, oracle, case):
+    """The fused layer entry point against its definition: numpy min/max, host fake quantization of both tensors,
+    the oracle's op on the fake-quantized tensors, bias_add, ReLU
+    (tf2/python/keras/layers/fake_approx_convolutional.py:223-261)."""
+    xs, fs, strides, use_bias, activation, (lo, hi) = case
+    rng = np.random.default_rng(xs[1] * 7 + fs[3])
+    x = rng.uniform(lo, hi, size=xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * 0.2).astype(np.float32)
+    bias = rng.uniform(-0.5, 0.5, size=fs[3]).astype(np.float32) if use_bias else None
+    table = pkg.synth.table_noisy(7)
+    layer = pkg.FakeApproxConv2D(strides, table, "same", activation=activation)
+    dev = gpu_util.dev()
+    y = layer(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev),
+              torch.from_numpy(bias).to(dev) if use_bias else None).cpu().numpy()
+    mm = (float(x.min()), float(x.max()), float(w.min()), float(w.max()))
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    rc, y_ref, _ = oracle.conv2d_fast(table, fq(x, mm[0], mm[1]), fq(w, mm[2], mm[3]), *mm, strides=strides,
+                                      padding="SAME", dilations=(1, 1))
+    assert rc == 0
+    if use_bias:
+        y_ref = (y_ref + bias).astype(np.float32)
+    if activation == "relu":
+        y_ref = np.maximum(y_ref, 0.0)
+    assert refimpl.linf_rel(y, y_ref) <= TOL
+
+
+def test_fake_approx_conv2d_layer_all_zero_input(pkg):
+    """min == max == 0 for the input: every quantization constant of that tensor is 0 (approx_ops_types.h:142-151)."""
+    dev = gpu_util.dev()
+    x = torch.zeros((1, 6, 6, 4), device=dev)
+    w = torch.from_numpy(np.random.default_rng(1).standard_normal((3, 3, 4, 8)).astype(np.float32)).to(dev)
+    y = pkg.FakeApproxConv2D((1, 1), pkg.synth.table_exact(), "same")(x, w)
+    assert torch.isfinite(y).all() and float(y.abs().max()) == 0.0

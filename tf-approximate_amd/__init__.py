@@ -6,6 +6,7 @@ The directory name is not a Python identifier; load the package with
 from . import fake_quant, synth  # noqa: F401
 from .ops import (  # noqa: F401
     ApproxConv2DWithMinMaxVars,
+    FakeApproxConv2D,
     InvalidArgumentError,
     TruthTable,
     UnimplementedError,

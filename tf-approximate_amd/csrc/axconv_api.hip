@@ -338,7 +338,7 @@ DensePlan make_plan(const ConvGeom &g, int cus)
 inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct DenseWorkspace {
-    size_t xq_off, psum_off, wq_off, fsum_off, part_off, total;
+    size_t xq_off, psum_off, wq_off, fsum_off, layer_off, part_off, total;
 };
 
 DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
@@ -349,6 +349,8 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
     w.psum_off = off; off += align_up((size_t)g.M * 4); // patch sums: one float per output pixel
     w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
     w.fsum_off = off; off += align_up((size_t)g.Co * 4);
+    w.layer_off = off;  // layer entry point: partial (min, max) pairs of both tensors, then the LayerQuant
+    off += align_up((size_t)4 * kMinMaxBlocks * sizeof(float)) + align_up(sizeof(LayerQuant));
     w.part_off = off;   // int32 partial sums of the K splits
     if (plan.k_splits > 1)
         off += align_up((size_t)plan.k_splits * (size_t)g.M * g.Co * 4);
@@ -389,10 +391,13 @@ enum class DenseOut { Float, AccI32 };
 int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *input, const float *filter,
               const uint8_t *input_codes, const uint8_t *filter_codes, int input_zero_code,
               float in_min, float in_max, float f_min, float f_max, float *out_f, int32_t *out_i,
-              void *workspace, size_t workspace_bytes, void *stream_v)
+              void *workspace, size_t workspace_bytes, void *stream_v, bool layer_mode = false,
+              const float *bias = nullptr, int activation = AXC_ACT_NONE)
 {
     if (!table || !desc)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
+    if (activation != AXC_ACT_NONE && activation != AXC_ACT_RELU)
+        return fail(AXC_INVALID_ARGUMENT, "unknown activation");
     PreparedDense pd;
     int rc = prepare_dense(desc, &pd);
     if (rc != AXC_OK)
@@ -434,21 +439,32 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     float *fsum = reinterpret_cast<float *>(ws + pd.ws.fsum_off);
 
     const uint32_t zp4 = phys_row((uint32_t)qp.input_zero_code) * 0x01010101u;
+    // by-value quantization of the two tensors (op entry points); the layer entry point computes its own on the device
+    TensorQuant tq_in = {qp.input_offset, qp.input_inv_scale, qp.input_scale, 0.0f, 0u, zp4};
+    TensorQuant tq_f = {qp.filter_offset, qp.filter_inv_scale, qp.filter_scale, 0.0f, 0u, 0u};
+    LayerQuant *lq_dev = nullptr;
+    if (layer_mode) {
+        ProfScope ps("layer_quant", stream);
+        float *partials = reinterpret_cast<float *>(ws + pd.ws.layer_off);
+        lq_dev = reinterpret_cast<LayerQuant *>(ws + pd.ws.layer_off + align_up((size_t)4 * kMinMaxBlocks * sizeof(float)));
+        AXC_HIP(launch_layer_quant(input, (int64_t)g.N * g.H * g.W * g.C, filter, (int64_t)g.K * g.Co, g.K, partials,
+                                   lq_dev, stream));
+    }
     if (codes_mode) {
         ProfScope ps("codes_relayout", stream);
         AXC_HIP(launch_codes_relayout(input_codes, g, zp4, xq, stream));
     } else {
         ProfScope ps("quantize_relayout", stream);
-        AXC_HIP(launch_quantize_relayout(input, g, qp.input_offset, qp.input_inv_scale, zp4, xq, nullptr, stream));
+        AXC_HIP(launch_quantize_relayout(input, g, tq_in, lq_dev, xq, nullptr, stream));
     }
     if (out_f && !codes_mode) {
         ProfScope ps("patch_sums", stream);
-        AXC_HIP(launch_patch_sums(input, g, psum, stream));
+        AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream));
     }
     {
         ProfScope ps("filter_pack", stream);
-        AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, g, pd.plan, qp.filter_offset,
-                                   qp.filter_inv_scale, wq, (out_f && !codes_mode) ? fsum : nullptr, stream));
+        AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, g, pd.plan, tq_f, lq_dev, wq,
+                                   (out_f && !codes_mode) ? fsum : nullptr, stream));
     }
 
     DenseParams p;
@@ -469,6 +485,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         p.k_m1xm2 = km;
     }
     p.zp4 = zp4;
+    p.lq_dev = lq_dev;
+    p.bias = bias;
+    p.relu = activation == AXC_ACT_RELU ? 1 : 0;
     p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
     p.wq_bytes = (uint32_t)((size_t)pd.plan.n_col_tiles * pd.plan.fills * 128);
     if (pd.plan.k_splits > 1) {
@@ -662,6 +681,16 @@ int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes)
         return rc;
     *bytes = pd.ws.total;
     return AXC_OK;
+}
+
+int axc_fake_approx_conv2d(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                           const float *filter, const float *bias, int activation, float *output, void *workspace,
+                           size_t workspace_bytes, void *stream)
+{
+    if (!output)
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    return run_dense(table, desc, input, filter, nullptr, nullptr, 0, 0.0f, 0.0f, 0.0f, 0.0f, output, nullptr, workspace,
+                     workspace_bytes, stream, true, bias, activation);
 }
 
 int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6])

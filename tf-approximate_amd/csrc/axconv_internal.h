@@ -43,6 +43,37 @@ struct DensePlan {
     int grid;
 };
 
+// Quantization of one tensor as the pre-pass kernels see it.
+struct TensorQuant {
+    float offset;       // nudged minimum
+    float inv_scale;
+    float scale;
+    float nudged_max;
+    uint32_t fq;        // 1: snap every value to the 8-bit grid first (the Keras layer's fake quantization)
+    uint32_t zp4;       // row-permuted code of 0.0f, replicated in all four bytes (input tensor only)
+};
+
+// Everything the kernels need to know about a layer's quantization.  The op entry points pass it by value
+// (min/max are host scalars there); the layer entry point computes it on the device from the tensors' own
+// min/max, so kernels take both a value and a device pointer and use the pointer when it is not null.
+struct LayerQuant {
+    TensorQuant in, flt;
+    float s1xs2, m1, m2, k_m1xm2;
+};
+
+// fake_quant_with_min_max_vars on one value (clamp to the nudged range, round half up to the grid), in the
+// float32 operations of TensorFlow's functor; identity unless q.fq.
+__device__ inline float fake_quant_value(float v, const TensorQuant &q)
+{
+    if (!q.fq)
+        return v;
+    if (q.scale == 0.0f)
+        return 0.0f;                       // min == max == 0: the whole tensor quantizes to 0
+    const float c = fmaxf(fminf(v, q.nudged_max), q.offset);
+    const float t = floorf(__fadd_rn(__fmul_rn(__fsub_rn(c, q.offset), q.inv_scale), 0.5f));
+    return __fadd_rn(__fmul_rn(t, q.scale), q.offset);
+}
+
 struct DenseParams {
     ConvGeom g;
     DensePlan plan;
@@ -57,6 +88,9 @@ struct DenseParams {
     float s1xs2, m1, m2, k_m1xm2; // epilogue constants; k_m1xm2 = float(K) * m1xM2
     uint32_t zp4;           // row-permuted zero code replicated in all four bytes
     uint32_t xq_bytes, wq_bytes; // sizes of the two streams (buffer-descriptor bounds)
+    const LayerQuant *lq_dev;    // not null: epilogue constants come from here instead of the four floats above
+    const float *bias;           // not null: added to every output column after the epilogue
+    int relu;                    // 1: max(x, 0) last
 };
 
 struct DepthwiseParams {
@@ -87,13 +121,17 @@ __device__ inline uint32_t quantize_code(float v, float offset, float inv_scale)
 }
 
 // ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
-hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
-                                    uint32_t zp4, uint32_t *xq, float *chsum, hipStream_t stream);
-hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream);
+hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
+                                    uint32_t *xq, float *chsum, hipStream_t stream);
+hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
+                             float *psum, hipStream_t stream);
+hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
+                              float *partials, LayerQuant *lq_dev, hipStream_t stream);
+constexpr int kMinMaxBlocks = 512;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch
 hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
                                  hipStream_t stream);
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
-                              const DensePlan &plan, float offset, float inv_scale,
+                              const DensePlan &plan, const TensorQuant &tq, const LayerQuant *lq_dev,
                               uint16_t *wq, float *fsum, hipStream_t stream);
 hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
                                 hipStream_t stream);

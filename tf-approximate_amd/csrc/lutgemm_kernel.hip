@@ -358,6 +358,14 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         // different 64-byte pieces of memory.  The wavefront therefore turns each of its wavefront-rows
         // through a private piece of LDS (every buffer is free after the last phase) so that NT/4 neighbouring
         // lanes write one pixel's NT columns: 16 or 8 contiguous runs per store instruction.
+        const float e_s1xs2 = p.lq_dev ? p.lq_dev->s1xs2 : p.s1xs2, e_m1 = p.lq_dev ? p.lq_dev->m1 : p.m1;
+        const float e_m2 = p.lq_dev ? p.lq_dev->m2 : p.m2, e_km = p.lq_dev ? p.lq_dev->k_m1xm2 : p.k_m1xm2;
+        // what the Keras layer does behind the op (bias_add, then the activation): fused into the store
+        auto finish = [&](float v, int col) {
+            if (p.bias)
+                v = __fadd_rn(v, p.bias[col]);
+            return p.relu ? fmaxf(v, 0.0f) : v;
+        };
         constexpr bool kTransposed = NT <= 32;
         if (kTransposed && (g.Co & 3) == 0) {
             constexpr int Q = NT / 4;                 // 16-byte quads (lanes) per pixel
@@ -371,7 +379,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 const int64_t m0 = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
                 const int nvalid = (int)(row_end - m0 < 64 ? row_end - m0 : 64);
                 const float psum = (!OUT_I32 && lane < nvalid) ? p.psum[m0 + lane] : 0.0f;
-                const float t1 = __fmul_rn(p.m2, psum);
+                const float t1 = __fmul_rn(e_m2, psum);
 #pragma unroll
                 for (int set = 0; set < SETS; ++set) {
                     const int h = (c0 + set) & (SETS - 1);
@@ -383,11 +391,11 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                         } else {
                             int col = ct * NT + h * 8 + e;
                             col = col < g.Co ? col : g.Co - 1;
-                            const float t0 = __fmul_rn((float)acc[r][set * 8 + e], p.s1xs2);
+                            const float t0 = __fmul_rn((float)acc[r][set * 8 + e], e_s1xs2);
                             const float t2 = __fadd_rn(t0, t1);
-                            const float t3 = __fmul_rn(p.m1, p.fsum[col]);
+                            const float t3 = __fmul_rn(e_m1, p.fsum[col]);
                             const float t4 = __fadd_rn(t2, t3);
-                            w[e] = __float_as_uint(__fsub_rn(t4, p.k_m1xm2));
+                            w[e] = __float_as_uint(finish(__fsub_rn(t4, e_km), col));
                         }
                     }
                     u32x4s lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
@@ -414,7 +422,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             const int64_t m = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64 + lane;
             // patch sum of the raw input in the reference's order (tap-major, channels ascending)
             const float psum = OUT_I32 ? 0.0f : p.psum[m];
-            const float t1 = __fmul_rn(p.m2, psum);
+            const float t1 = __fmul_rn(e_m2, psum);
 #pragma unroll
             for (int set = 0; set < SETS; ++set) {
                 const int h = (c0 + set) & (SETS - 1);
@@ -441,11 +449,11 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         const int col = col0 + e < g.Co ? col0 + e : g.Co - 1;
-                        const float t0 = __fmul_rn((float)acc[r][set * 8 + e], p.s1xs2);
+                        const float t0 = __fmul_rn((float)acc[r][set * 8 + e], e_s1xs2);
                         const float t2 = __fadd_rn(t0, t1);
-                        const float t3 = __fmul_rn(p.m1, p.fsum[col]);
+                        const float t3 = __fmul_rn(e_m1, p.fsum[col]);
                         const float t4 = __fadd_rn(t2, t3);
-                        v[e] = __fsub_rn(t4, p.k_m1xm2);
+                        v[e] = finish(__fsub_rn(t4, e_km), col);
                     }
                     if (vec) {
                         *reinterpret_cast<float4 *>(p.out_f + o) = make_float4(v[0], v[1], v[2], v[3]);

@@ -11,10 +11,13 @@ namespace axc {
 //   chsum[N][H][W]      sum over channels of the raw floats, c ascending
 // One thread per pixel: the channel loop is sequential so the sum has the reference's order within a pixel.
 __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__restrict__ x, int64_t pixels,
-                                                                 int H, int W, int C, int C4, float offset,
-                                                                 float inv_scale, uint32_t *__restrict__ xq,
-                                                                 float *__restrict__ chsum, uint32_t zp4)
+                                                                 int H, int W, int C, int C4, const TensorQuant tq,
+                                                                 const LayerQuant *__restrict__ lq_dev,
+                                                                 uint32_t *__restrict__ xq,
+                                                                 float *__restrict__ chsum)
 {
+    const TensorQuant q = lq_dev ? lq_dev->in : tq;
+    const uint32_t zp4 = q.zp4;
     const int64_t pix = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     // the extra [C4][W] row behind the image rows: every dword is the zero-point code x4
     for (int64_t i = pix; i < (int64_t)C4 * W; i += (int64_t)gridDim.x * blockDim.x)
@@ -31,9 +34,9 @@ __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__r
         for (int i = 0; i < 4; ++i) {
             const int c = c4 * 4 + i;
             if (c < C) {
-                const float v = src[c];
+                const float v = fake_quant_value(src[c], q);
                 sum = __fadd_rn(sum, v);
-                packed |= phys_row(quantize_code(v, offset, inv_scale)) << (8 * i);
+                packed |= phys_row(quantize_code(v, q.offset, q.inv_scale)) << (8 * i);
             }
         }
         xq[(nh * C4 + c4) * W + w] = packed;
@@ -45,9 +48,12 @@ __global__ void __launch_bounds__(256) quantize_relayout_kernel(const float *__r
 // Same result as quantize_relayout_kernel for C % 4 == 0, with fully coalesced reads: consecutive lanes
 // read consecutive float4 of the NHWC input (one float4 = the four channels of one xq dword).
 __global__ void __launch_bounds__(256) quantize_relayout_vec4_kernel(const float4 *__restrict__ x4, int64_t quads,
-                                                                      int W, int C4, float offset, float inv_scale,
-                                                                      uint32_t *__restrict__ xq, uint32_t zp4)
+                                                                      int W, int C4, const TensorQuant tq,
+                                                                      const LayerQuant *__restrict__ lq_dev,
+                                                                      uint32_t *__restrict__ xq)
 {
+    const TensorQuant q = lq_dev ? lq_dev->in : tq;
+    const uint32_t zp4 = q.zp4;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     // the extra [C4][W] row behind the image rows: every dword is the zero-point code x4
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (int64_t)C4 * W; i += stride)
@@ -58,10 +64,10 @@ __global__ void __launch_bounds__(256) quantize_relayout_vec4_kernel(const float
         const int c4 = (int)(i - pix * C4);
         const int64_t nh = pix / W;
         const int w = (int)(pix - nh * W);
-        const uint32_t packed = phys_row(quantize_code(v.x, offset, inv_scale)) |
-                                (phys_row(quantize_code(v.y, offset, inv_scale)) << 8) |
-                                (phys_row(quantize_code(v.z, offset, inv_scale)) << 16) |
-                                (phys_row(quantize_code(v.w, offset, inv_scale)) << 24);
+        const uint32_t packed = phys_row(quantize_code(fake_quant_value(v.x, q), q.offset, q.inv_scale)) |
+                                (phys_row(quantize_code(fake_quant_value(v.y, q), q.offset, q.inv_scale)) << 8) |
+                                (phys_row(quantize_code(fake_quant_value(v.z, q), q.offset, q.inv_scale)) << 16) |
+                                (phys_row(quantize_code(fake_quant_value(v.w, q), q.offset, q.inv_scale)) << 24);
         xq[(nh * C4 + c4) * W + w] = packed;
     }
 }
@@ -71,9 +77,17 @@ __global__ void __launch_bounds__(256) quantize_relayout_vec4_kernel(const float
 // (kh, kw, c ascending; taps outside the image add 0.0f, which leaves the sum unchanged).  fp32 addition is
 // not associative and this sum is multiplied by the filter offset in the epilogue, so any other order
 // shows up in the output at the 1e-4 level for inputs with a large mean.  One thread per output pixel.
-__global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict__ x, ConvGeom g,
+__device__ __forceinline__ float4 fake_quant_value4(float4 v, const TensorQuant &q)
+{
+    return make_float4(fake_quant_value(v.x, q), fake_quant_value(v.y, q), fake_quant_value(v.z, q),
+                       fake_quant_value(v.w, q));
+}
+
+__global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict__ x, ConvGeom g, const TensorQuant tq,
+                                                          const LayerQuant *__restrict__ lq_dev,
                                                           float *__restrict__ psum)
 {
+    const TensorQuant q = lq_dev ? lq_dev->in : tq;
     const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (m >= g.M)
         return;
@@ -94,7 +108,7 @@ __global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict
             if ((g.C & 3) == 0) {
                 const float4 *src4 = reinterpret_cast<const float4 *>(src);
                 for (int c4 = 0; c4 < g.C / 4; ++c4) {
-                    const float4 v = src4[c4];
+                    const float4 v = fake_quant_value4(src4[c4], q);
                     s = __fadd_rn(s, v.x);
                     s = __fadd_rn(s, v.y);
                     s = __fadd_rn(s, v.z);
@@ -102,7 +116,7 @@ __global__ void __launch_bounds__(256) patch_sums_kernel(const float *__restrict
                 }
             } else {
                 for (int c = 0; c < g.C; ++c)
-                    s = __fadd_rn(s, src[c]);
+                    s = __fadd_rn(s, fake_quant_value(src[c], q));
             }
         }
     }
@@ -120,8 +134,11 @@ constexpr int kPsRow = kPsCh + 4; // padded row (floats): conflict-free 16-byte 
 constexpr int kPsLoads = kPsCh / 4 * kPsTile / kPsTile; // float4 loads per thread per slice
 
 __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *__restrict__ x, ConvGeom g,
+                                                                    const TensorQuant tq,
+                                                                    const LayerQuant *__restrict__ lq_dev,
                                                                     float *__restrict__ psum)
 {
+    const TensorQuant qt = lq_dev ? lq_dev->in : tq;
     __shared__ int pix_base[kPsTile];  // (n * H) of the pixel's image, or -1 when the pixel does not exist
     __shared__ int pix_hw[kPsTile];    // input row / column of tap (0, 0), 16 bits each
     __shared__ __align__(16) float tile[kPsTile * kPsRow];
@@ -163,7 +180,8 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
             const int ih = lih[i] + kh * g.dh, iw = liw[i] + kw * g.dw;
             v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (lbase[i] >= 0 && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && c0 + j * 4 < g.C)
-                v[i] = *reinterpret_cast<const float4 *>(x + ((int64_t)(lbase[i] + ih) * g.W + iw) * g.C + c0 + j * 4);
+                v[i] = fake_quant_value4(
+                    *reinterpret_cast<const float4 *>(x + ((int64_t)(lbase[i] + ih) * g.W + iw) * g.C + c0 + j * 4), qt);
         }
     };
     float s = 0.0f;
@@ -198,8 +216,11 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
 // about once (plus the halo) instead of once per filter tap; the sequential chains then read LDS only.
 // Pixels are padded to C + 4 floats so that the 16-byte reads of neighbouring threads fall into different banks.
 __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, ConvGeom g, int rb,
-                                                                int in_rows, float *__restrict__ psum)
+                                                                int in_rows, const TensorQuant tq,
+                                                                const LayerQuant *__restrict__ lq_dev,
+                                                                float *__restrict__ psum)
 {
+    const TensorQuant qt = lq_dev ? lq_dev->in : tq;
     extern __shared__ __align__(16) unsigned char ps_lds[];
     float *const rows = reinterpret_cast<float *>(ps_lds);
     const int t = threadIdx.x;
@@ -218,7 +239,7 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
             for (int w = w0; w < g.W; w += wstep) {
                 float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 if (inb)
-                    v = *reinterpret_cast<const float4 *>(src + (int64_t)w * g.C);
+                    v = fake_quant_value4(*reinterpret_cast<const float4 *>(src + (int64_t)w * g.C), qt);
                 *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
             }
         }
@@ -231,7 +252,8 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
             const int ih = ih_first + r;
             float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if ((unsigned)ih < (unsigned)g.H)
-                v = *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + w) * g.C + q * 4);
+                v = fake_quant_value4(
+                    *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + w) * g.C + q * 4), qt);
             *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
         }
     }
@@ -290,8 +312,8 @@ __global__ void __launch_bounds__(256) codes_relayout_kernel(const uint8_t *__re
 //   channel = q*4 + sub*KS + kk, column = ct*NT + j; kNullWeight where channel >= C or column >= Co.
 __device__ __forceinline__ void filter_pack_element(const int64_t i, const float *__restrict__ filter,
                                                     const uint8_t *__restrict__ filter_codes, int taps, int C,
-                                                    int C4, int Co, int nt, int n_col_tiles, float offset,
-                                                    float inv_scale, uint16_t *__restrict__ wq)
+                                                    int C4, int Co, int nt, int n_col_tiles, const TensorQuant &qf,
+                                                    uint16_t *__restrict__ wq)
 {
     const int ks = 64 / nt, subs = 4 / ks;
     const int fills = taps * C4 * subs;
@@ -313,7 +335,7 @@ __device__ __forceinline__ void filter_pack_element(const int64_t i, const float
     if (c < C && col < Co) {
         const int64_t idx = ((int64_t)tap * C + c) * Co + col;
         code = filter_codes ? (uint16_t)filter_codes[idx]
-                            : (uint16_t)quantize_code(filter[idx], offset, inv_scale);
+                            : (uint16_t)quantize_code(fake_quant_value(filter[idx], qf), qf.offset, qf.inv_scale);
     }
     wq[i] = code;
 }
@@ -329,7 +351,7 @@ constexpr int kFsLdsBytes = kFsRows * 65 * 4;
 extern __shared__ __align__(16) unsigned char fs_lds[];
 
 __device__ __forceinline__ void filter_sums_block(const int block, const float *__restrict__ filter, int K, int Co,
-                                                  float *__restrict__ fsum)
+                                                  const TensorQuant &q, float *__restrict__ fsum)
 {
     constexpr int kBatch = 32, kPer = kFsRows * 64 / kFsThreads; // loads per thread per pass
     float *const stage = reinterpret_cast<float *>(fs_lds);
@@ -342,7 +364,7 @@ __device__ __forceinline__ void filter_sums_block(const int block, const float *
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
             const int k = k0 + rsub + i * (kFsThreads / 64);
-            v[i] = (k < K && col0 + cl < Co) ? filter[(int64_t)k * Co + col0 + cl] : 0.0f;
+            v[i] = (k < K && col0 + cl < Co) ? fake_quant_value(filter[(int64_t)k * Co + col0 + cl], q) : 0.0f;
         }
         __syncthreads(); // previous pass consumed
 #pragma unroll
@@ -374,16 +396,18 @@ __device__ __forceinline__ void filter_sums_block(const int block, const float *
 __global__ void __launch_bounds__(kFsThreads) filter_prep_kernel(const float *__restrict__ filter,
                                                                   const uint8_t *__restrict__ filter_codes, int taps,
                                                                   int C, int C4, int Co, int nt, int n_col_tiles,
-                                                                  float offset, float inv_scale,
+                                                                  const TensorQuant tq,
+                                                                  const LayerQuant *__restrict__ lq_dev,
                                                                   uint16_t *__restrict__ wq, int sum_blocks,
                                                                   float *__restrict__ fsum)
 {
+    const TensorQuant q = lq_dev ? lq_dev->flt : tq;
     if ((int)blockIdx.x < sum_blocks) {
-        filter_sums_block((int)blockIdx.x, filter, taps * C, Co, fsum);
+        filter_sums_block((int)blockIdx.x, filter, taps * C, Co, q, fsum);
         return;
     }
     const int64_t i = (int64_t)(blockIdx.x - sum_blocks) * blockDim.x + threadIdx.x;
-    filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, offset, inv_scale, wq);
+    filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, q, wq);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -422,6 +446,119 @@ __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t *__restrict__ ds
         dst[i] = value;
 }
 
+// ---- the Keras layer's pre-step: per-tensor min / max and the quantization constants, all on the device ----
+// (tf2/python/keras/layers/fake_approx_convolutional.py:233-242: reduce_min / reduce_max of the batch and of
+// the kernel, then fake quantization with them.)  Stage 1: one (min, max) pair per workgroup.
+__global__ void __launch_bounds__(256) minmax_partial_kernel(const float *__restrict__ v, int64_t n,
+                                                              float *__restrict__ partials)
+{
+    __shared__ float smin[256], smax[256];
+    float lo = INFINITY, hi = -INFINITY;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const float x = v[i];
+        lo = fminf(lo, x);
+        hi = fmaxf(hi, x);
+    }
+    smin[threadIdx.x] = lo;
+    smax[threadIdx.x] = hi;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) {
+            smin[threadIdx.x] = fminf(smin[threadIdx.x], smin[threadIdx.x + s]);
+            smax[threadIdx.x] = fmaxf(smax[threadIdx.x], smax[threadIdx.x + s]);
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partials[2 * blockIdx.x] = smin[0];
+        partials[2 * blockIdx.x + 1] = smax[0];
+    }
+}
+
+// Nudge + UpdateVarQuantProps (tf2/src/approx_ops_types.h:29-49,135-152) for one tensor, every operation rounded
+// on its own like the host code of axc_quant_props_compute.
+__device__ void tensor_quant_device(float mn, float mx, TensorQuant *t, int *zero_point)
+{
+    t->fq = 1u;
+    t->zp4 = 0u;
+    *zero_point = 0;
+    if (mn == 0.0f && mx == 0.0f) {
+        t->offset = t->inv_scale = t->scale = t->nudged_max = 0.0f;
+        return;
+    }
+    const float sc = __fdiv_rn(__fsub_rn(mx, mn), 255.0f);
+    const float zp_from_min = __fsub_rn(0.0f, __fdiv_rn(mn, sc));
+    int zp;
+    if (zp_from_min < 0.0f)
+        zp = 0;
+    else if (zp_from_min > 255.0f)
+        zp = 255;
+    else
+        zp = (int)(uint16_t)roundf(zp_from_min);
+    t->scale = sc;
+    t->offset = __fmul_rn(__fsub_rn(0.0f, (float)zp), sc);
+    t->nudged_max = __fmul_rn(__fsub_rn(255.0f, (float)zp), sc);
+    t->inv_scale = __fdiv_rn(1.0f, sc);
+    *zero_point = zp;
+}
+
+// Stage 2: one workgroup folds the partial pairs of both tensors and writes the layer's constants.
+__global__ void __launch_bounds__(256) layer_quant_kernel(const float *__restrict__ partials, int n_in, int n_flt,
+                                                           int K, LayerQuant *__restrict__ out)
+{
+    __shared__ float red[4][256];
+    float v[4] = {INFINITY, -INFINITY, INFINITY, -INFINITY};
+    for (int i = threadIdx.x; i < n_in; i += 256) {
+        v[0] = fminf(v[0], partials[2 * i]);
+        v[1] = fmaxf(v[1], partials[2 * i + 1]);
+    }
+    const float *pf = partials + 2 * kMinMaxBlocks;
+    for (int i = threadIdx.x; i < n_flt; i += 256) {
+        v[2] = fminf(v[2], pf[2 * i]);
+        v[3] = fmaxf(v[3], pf[2 * i + 1]);
+    }
+    for (int k = 0; k < 4; ++k)
+        red[k][threadIdx.x] = v[k];
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s)
+            for (int k = 0; k < 4; ++k)
+                red[k][threadIdx.x] = (k & 1) ? fmaxf(red[k][threadIdx.x], red[k][threadIdx.x + s])
+                                              : fminf(red[k][threadIdx.x], red[k][threadIdx.x + s]);
+        __syncthreads();
+    }
+    if (threadIdx.x != 0)
+        return;
+    LayerQuant lq;
+    int zp_in = 0, zp_f = 0;
+    tensor_quant_device(red[0][0], red[1][0], &lq.in, &zp_in);
+    tensor_quant_device(red[2][0], red[3][0], &lq.flt, &zp_f);
+    // the code the op gives 0.0f (what taps outside the image look up): its own quantize expression
+    lq.in.zp4 = phys_row(quantize_code(0.0f, lq.in.offset, lq.in.inv_scale)) * 0x01010101u;
+    // approx_ops_types.h:184-187
+    lq.s1xs2 = __fmul_rn(lq.in.scale, lq.flt.scale);
+    lq.m1 = lq.in.offset;
+    lq.m2 = lq.flt.offset;
+    lq.k_m1xm2 = __fmul_rn((float)K, __fmul_rn(lq.in.offset, lq.flt.offset));
+    *out = lq;
+}
+
+hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
+                              float *partials, LayerQuant *lq_dev, hipStream_t stream)
+{
+    auto blocks = [](int64_t n) {
+        const int64_t b = (n + 256 * 16 - 1) / (256 * 16);
+        return (int)(b < 1 ? 1 : (b > kMinMaxBlocks ? kMinMaxBlocks : b));
+    };
+    const int b_in = blocks(n_input), b_f = blocks(n_filter);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(b_in), dim3(256), 0, stream, input, n_input, partials);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(b_f), dim3(256), 0, stream, filter, n_filter,
+                       partials + 2 * kMinMaxBlocks);
+    hipLaunchKernelGGL(layer_quant_kernel, dim3(1), dim3(256), 0, stream, partials, b_in, b_f, K, lq_dev);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t stream)
 {
     for (int64_t done = 0; done < n; done += (int64_t)1 << 30) { // int-sized pieces
@@ -437,9 +574,18 @@ template <int V>
 __global__ void __launch_bounds__(256) splitk_epilogue_kernel(const int32_t *__restrict__ part, int ks, int64_t mc,
                                                                int Co, const float *__restrict__ psum,
                                                                const float *__restrict__ fsum, float s1xs2, float m1,
-                                                               float m2, float k_m1xm2, float *__restrict__ out_f,
+                                                               float m2, float k_m1xm2,
+                                                               const LayerQuant *__restrict__ lq_dev,
+                                                               const float *__restrict__ bias, int relu,
+                                                               float *__restrict__ out_f,
                                                                int32_t *__restrict__ out_i)
 {
+    if (lq_dev) {
+        s1xs2 = lq_dev->s1xs2;
+        m1 = lq_dev->m1;
+        m2 = lq_dev->m2;
+        k_m1xm2 = lq_dev->k_m1xm2;
+    }
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
     if (i >= mc)
         return;
@@ -472,6 +618,10 @@ __global__ void __launch_bounds__(256) splitk_epilogue_kernel(const int32_t *__r
         const float t3 = __fmul_rn(m1, fsum[col + e]);
         const float t4 = __fadd_rn(t2, t3);
         r[e] = __fsub_rn(t4, k_m1xm2);
+        if (bias)
+            r[e] = __fadd_rn(r[e], bias[col + e]);
+        if (relu)
+            r[e] = fmaxf(r[e], 0.0f);
     }
     if (V == 4)
         *reinterpret_cast<float4 *>(out_f + i) = make_float4(r[0], r[1 % V], r[2 % V], r[3 % V]);
@@ -485,10 +635,12 @@ hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials,
     const int64_t mc = p.g.M * p.g.Co;
     if ((p.g.Co & 3) == 0)
         hipLaunchKernelGGL(splitk_epilogue_kernel<4>, dim3(blocks_for(mc / 4, 256)), dim3(256), 0, stream, partials,
-                           p.plan.k_splits, mc, p.g.Co, p.psum, p.fsum, p.s1xs2, p.m1, p.m2, p.k_m1xm2, out_f, out_i);
+                           p.plan.k_splits, mc, p.g.Co, p.psum, p.fsum, p.s1xs2, p.m1, p.m2, p.k_m1xm2, p.lq_dev, p.bias, p.relu,
+                           out_f, out_i);
     else
         hipLaunchKernelGGL(splitk_epilogue_kernel<1>, dim3(blocks_for(mc, 256)), dim3(256), 0, stream, partials,
-                           p.plan.k_splits, mc, p.g.Co, p.psum, p.fsum, p.s1xs2, p.m1, p.m2, p.k_m1xm2, out_f, out_i);
+                           p.plan.k_splits, mc, p.g.Co, p.psum, p.fsum, p.s1xs2, p.m1, p.m2, p.k_m1xm2, p.lq_dev, p.bias, p.relu,
+                           out_f, out_i);
     return hipGetLastError();
 }
 
@@ -500,8 +652,8 @@ static hipError_t launch_zero_point_row(const ConvGeom &g, uint32_t zp4, uint32_
     return hipGetLastError();
 }
 
-hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float offset, float inv_scale,
-                                    uint32_t zp4, uint32_t *xq, float *chsum, hipStream_t stream)
+hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
+                                    uint32_t *xq, float *chsum, hipStream_t stream)
 {
     const int64_t pixels = (int64_t)g.N * g.H * g.W;
     if ((g.C & 3) == 0 && !chsum && ((uintptr_t)x & 15) == 0) {
@@ -509,15 +661,16 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, float off
         int64_t blocks = (quads + 256 * 4 - 1) / (256 * 4);
         if (blocks > 65536) blocks = 65536;
         hipLaunchKernelGGL(quantize_relayout_vec4_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           reinterpret_cast<const float4 *>(x), quads, g.W, g.C4, offset, inv_scale, xq, zp4);
+                           reinterpret_cast<const float4 *>(x), quads, g.W, g.C4, tq, lq_dev, xq);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(quantize_relayout_kernel, dim3(blocks_for(pixels, 256)), dim3(256), 0, stream, x, pixels,
-                       g.H, g.W, g.C, g.C4, offset, inv_scale, xq, chsum, zp4);
+                       g.H, g.W, g.C, g.C4, tq, lq_dev, xq, chsum);
     return hipGetLastError();
 }
 
-hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hipStream_t stream)
+hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
+                             float *psum, hipStream_t stream)
 {
     const bool vec = (g.C & 3) == 0 && ((uintptr_t)x & 15) == 0;
     if (vec && g.OW <= 1024) {
@@ -544,15 +697,15 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, float *psum, hip
                 return e;
             const int bands = (g.OH + rb - 1) / rb;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(g.N * bands)), dim3(threads), lds, stream, x, g,
-                               rb, in_rows, psum);
+                               rb, in_rows, tq, lq_dev, psum);
             return hipGetLastError();
         }
     }
     if (vec)
         hipLaunchKernelGGL(patch_sums_tiled_kernel, dim3(blocks_for(g.M, kPsTile)), dim3(kPsTile), 0, stream, x, g,
-                           psum);
+                           tq, lq_dev, psum);
     else
-        hipLaunchKernelGGL(patch_sums_kernel, dim3(blocks_for(g.M, 256)), dim3(256), 0, stream, x, g, psum);
+        hipLaunchKernelGGL(patch_sums_kernel, dim3(blocks_for(g.M, 256)), dim3(256), 0, stream, x, g, tq, lq_dev, psum);
     return hipGetLastError();
 }
 
@@ -569,8 +722,8 @@ hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32
 }
 
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
-                              const DensePlan &plan, float offset, float inv_scale, uint16_t *wq, float *fsum,
-                              hipStream_t stream)
+                              const DensePlan &plan, const TensorQuant &tq, const LayerQuant *lq_dev, uint16_t *wq,
+                              float *fsum, hipStream_t stream)
 {
     const int64_t total = (int64_t)plan.n_col_tiles * plan.fills * 64;
     const int sum_blocks = (fsum && filter) ? (int)blocks_for(g.Co, 64) : 0;
@@ -582,8 +735,8 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
             return ea;
     }
     hipLaunchKernelGGL(filter_prep_kernel, dim3(sum_blocks + blocks_for(total, kFsThreads)), dim3(kFsThreads), lds,
-                       stream, filter, filter_codes, g.KH * g.KW, g.C, g.C4, g.Co, plan.nt, plan.n_col_tiles, offset,
-                       inv_scale, wq, sum_blocks, fsum);
+                       stream, filter, filter_codes, g.KH * g.KW, g.C, g.C4, g.Co, plan.nt, plan.n_col_tiles, tq, lq_dev,
+                       wq, sum_blocks, fsum);
     return hipGetLastError();
 }
 

@@ -43,7 +43,11 @@ class ApproxNetwork:
     """A forward pass described as a small program over named tensors:
     ("conv", dst, src, ConvSpec) | ("add_relu", dst, a, b) | ("maxpool", dst, src)"""
 
-    def __init__(self, program, input_shape, table, seed=0, device="cuda:0"):
+    def __init__(self, program, input_shape, table, seed=0, device="cuda:0", fused_layers=False):
+        """fused_layers: run every dense convolution through the layer entry point (min/max of each batch and
+        fake quantization computed on the device, ReLU fused), as the reference's Keras layer does per call;
+        otherwise ranges come from a calibration pass and the plain op runs."""
+        self.fused_layers = fused_layers
         self.program = program
         self.input_shape = tuple(input_shape)
         self.device = torch.device(device)
@@ -56,8 +60,12 @@ class ApproxNetwork:
             spec = step[3]
             w = _he_normal(rng, spec.filter_shape())
             self.weights[i] = torch.from_numpy(w).to(self.device)
-            self.ops[i] = ops.ApproxConv2DWithMinMaxVars([1, spec.stride, spec.stride, 1], 8, self.table, "SAME",
-                                                         depthwise=spec.depthwise)
+            if fused_layers and not spec.depthwise:
+                self.ops[i] = ops.FakeApproxConv2D((spec.stride, spec.stride), self.table, "SAME",
+                                                   activation="relu" if spec.relu else None)
+            else:
+                self.ops[i] = ops.ApproxConv2DWithMinMaxVars([1, spec.stride, spec.stride, 1], 8, self.table, "SAME",
+                                                             depthwise=spec.depthwise)
 
     def conv_count(self):
         return len(self.ops)
@@ -72,7 +80,14 @@ class ApproxNetwork:
             if kind == "conv":
                 src, spec = t[step[2]], step[3]
                 w = self.weights[i]
-                if calibrate:
+                if self.fused_layers and not spec.depthwise:
+                    y = self.ops[i](src, w)
+                    if trace is not None:
+                        trace.append((spec, src.cpu().numpy(), w.cpu().numpy(), None, y.cpu().numpy()))
+                    macs += spec.macs(y.shape[1], y.shape[2], y.shape[0])
+                    t[dst] = y
+                    continue
+                if calibrate or i not in self.ranges:
                     lo, hi = torch.aminmax(src)
                     wlo, whi = torch.aminmax(w)
                     self.ranges[i] = (float(lo), float(hi), float(wlo), float(whi))
@@ -143,9 +158,9 @@ NETWORKS = {
 }
 
 
-def build(name, table, seed=0, device="cuda:0"):
+def build(name, table, seed=0, device="cuda:0", fused_layers=False):
     builder, shape, (lo, hi) = NETWORKS[name]
-    net = ApproxNetwork(builder(), shape, table, seed=seed, device=device)
+    net = ApproxNetwork(builder(), shape, table, seed=seed, device=device, fused_layers=fused_layers)
     rng = np.random.default_rng(seed + 1)
     x = torch.from_numpy(rng.uniform(lo, hi, size=shape).astype(np.float32)).to(net.device)
     return net, x

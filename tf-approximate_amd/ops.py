@@ -192,6 +192,40 @@ class ApproxConv2DWithMinMaxVars:
         return self._run(input, filter, (input_min, input_max, filter_min, filter_max), True)
 
 
+class FakeApproxConv2D:
+    """The reference's Keras layer around the op (FakeApproxConv2D.call,
+    tf2/python/keras/layers/fake_approx_convolutional.py:223-261) as one device-side call: min/max of the batch
+    and of the kernel, fake quantization of both, the op, bias_add, activation.  No host synchronisation."""
+
+    def __init__(self, strides, mul_map_file, padding="SAME", dilation_rate=(1, 1), activation=None, num_bits=8):
+        if activation not in (None, "relu"):
+            raise UnimplementedError("activation %r: only None and 'relu' are fused" % (activation,))
+        self.op = ApproxConv2DWithMinMaxVars([1, strides[0], strides[1], 1], num_bits, mul_map_file, padding.upper(),
+                                             dilations=[1, dilation_rate[0], dilation_rate[1], 1])
+        self.activation = 1 if activation == "relu" else 0
+
+    def __call__(self, inputs, kernel, bias=None):
+        lib = _lib.load()
+        inputs = _require_device_f32(inputs, "input")
+        kernel = _require_device_f32(kernel, "filter")
+        if bias is not None:
+            bias = _require_device_f32(bias, "bias")
+            if bias.numel() != kernel.shape[3]:
+                raise InvalidArgumentError("bias must have one value per output channel")
+        desc = self.op._desc(inputs, kernel)
+        dims = conv2d_geometry(desc)
+        nbytes = ctypes.c_size_t()
+        _check(lib.axc_conv2d_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+        ws = _workspace(inputs.device, nbytes.value)
+        out = torch.empty(self.op._out_shape(dims), dtype=torch.float32, device=inputs.device)
+        with torch.cuda.device(inputs.device):
+            _check(lib.axc_fake_approx_conv2d(self.op.table.handle, ctypes.byref(desc), inputs.data_ptr(),
+                                              kernel.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                              self.activation, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                              _stream_ptr(inputs.device)))
+        return out
+
+
 def conv2d_tile_plan(input_shape, filter_shape, strides=(1, 1, 1, 1), padding="SAME", dilations=(1, 1, 1, 1)):
     """The dense kernel's tile plan for a layer on the current device, as a dict."""
     lib = _lib.load()
