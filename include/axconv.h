@@ -107,6 +107,21 @@ int axc_fake_approx_conv2d(const axc_table *table, const axc_conv2d_desc *desc, 
                            const float *filter, const float *bias, int activation, float *output, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* The tf1 integer op AxConv2D (tf1/axqconv/axqconv.cc:66-94 registration, :113-278 ReferenceAxConvFunctor,
+ * :286-441 AxQuantizedConv2DOp): quint8 input and filter codes in, qint32 out,
+ *   out = sum over the patch of  T[a][b] - a*offset_filter - b*offset_input + offset_input*offset_filter,
+ * taps outside the image reading a = offset_input; padding origin by that functor's own rule (:153-163).
+ * offset_* are what the reference derives with FloatToQuantizedUnclamped(0, min, max) (TensorFlow, third party).
+ * Strides must be equal, dilations 1.  Workspace: axc_conv2d_workspace_bytes. */
+int axc_axconv2d_quint8(const axc_table *table, const axc_conv2d_desc *desc, const uint8_t *input,
+                        const uint8_t *filter, int32_t offset_input, int32_t offset_filter, int32_t *output,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+/* AxTune of ApproximateSelector::init (tf1/axqconv/approximate_selector.h:52-85), host side: tuned[i][w] =
+ * table[i][w2(w)] with w2 the weight whose column is closest to exact multiplication by w.  table and tuned are
+ * uint16[65536] in host memory and may be the same buffer. */
+int axc_table_tune_weights(const uint16_t *table, uint16_t *tuned);
+
 /* How the dense kernel would cut this layer on the current device (for tools and tests; the reference has no
  * counterpart, its launch shapes are fixed in cuda/approx_nn_conv_kernels.cu:296-627):
  * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups }. */

@@ -576,3 +576,58 @@ double axo_time_reference_chunk(const uint16_t *table, axo_conv_desc *d,
     free(filter_coeff);
     return t1 - t0;
 }
+
+/* tf1/axqconv/axqconv.cc:113-278 */
+void axo_axconv2d_tf1(const uint16_t *table, const uint8_t *input, int batches, int in_h, int in_w, int in_depth,
+                      int input_offset, const uint8_t *filter, int filter_h, int filter_w, int filter_count,
+                      int filter_offset, int stride, int padding, int32_t *output, int out_h, int out_w)
+{
+    int left, top;
+    if (padding == AXO_PAD_VALID) { /* :153-157 */
+        left = ((out_w - 1) * stride + filter_w - in_w + 1) / 2;
+        top = ((out_h - 1) * stride + filter_h - in_h + 1) / 2;
+    } else {                        /* :158-163 */
+        left = ((out_w - 1) * stride + filter_w - in_w) / 2;
+        top = ((out_h - 1) * stride + filter_h - in_h) / 2;
+    }
+    for (int batch = 0; batch < batches; ++batch)
+        for (int oy = 0; oy < out_h; ++oy)
+            for (int ox = 0; ox < out_w; ++ox)
+                for (int oc = 0; oc < filter_count; ++oc) {
+                    const int x0 = ox * stride - left, y0 = oy * stride - top;
+                    int32_t total = 0;
+                    for (int fy = 0; fy < filter_h; ++fy)
+                        for (int fx = 0; fx < filter_w; ++fx)
+                            for (int ic = 0; ic < in_depth; ++ic) {
+                                const int ix = x0 + fx, iy = y0 + fy;
+                                int32_t a;
+                                if (ix >= 0 && ix < in_w && iy >= 0 && iy < in_h)
+                                    a = input[(((size_t)batch * in_h + iy) * in_w + ix) * in_depth + ic];
+                                else
+                                    a = (uint8_t)input_offset; /* :215: stored into the quint8 source value */
+                                const int32_t b = filter[(((size_t)fy * filter_w + fx) * in_depth + ic) * filter_count + oc];
+                                const int32_t axm = table[a * 256 + b];
+                                total += axm - a * filter_offset - b * input_offset + input_offset * filter_offset;
+                            }
+                    output[(((size_t)batch * out_h + oy) * out_w + ox) * filter_count + oc] = total;
+                }
+}
+
+/* tf1/axqconv/approximate_selector.h:52-85 */
+void axo_table_tune_weights(const uint16_t *table, uint16_t *tuned)
+{
+    for (int w = 0; w < 256; ++w) {
+        int wpos = -1, werr = 0;
+        for (int w2 = 0; w2 < 256; ++w2) {
+            int sumerr = 0;
+            for (int i = 0; i < 256; ++i)
+                sumerr += abs(i * w - (int)table[i * 256 + w2]);
+            if (sumerr < werr || (werr == sumerr && w2 == w) || wpos < 0) {
+                werr = sumerr;
+                wpos = w2;
+            }
+        }
+        for (int i = 0; i < 256; ++i)
+            tuned[i * 256 + w] = table[i * 256 + wpos];
+    }
+}

@@ -17,6 +17,8 @@
  *   axo_im2col / axo_gemm_table / axo_gemm_combined / axo_conv2d
  *                                       brute force, integer matmul with the exact table,
  *                                       conv2d(fq(X), fq(F)) by a library routine, direct 7-loop form
+ *   axo_axconv2d_tf1                    exact table => integer convolution of (code - offset) by numpy
+ *   axo_table_tune_weights              exact table is a fixed point; brute-force argmin in numpy
  *   axo_depthwise_conv2d                no counterpart in the reference (it rejects grouped convolutions);
  *                                       defined here as the dense op applied per channel
  */
@@ -129,6 +131,19 @@ double axo_time_reference_chunk(const uint16_t *table, axo_conv_desc *d,
                                 const float *input, const float *filter,
                                 float in_min, float in_max, float f_min, float f_max,
                                 int patches, float *out_chunk);
+
+/* tf1 AxConv2D, ReferenceAxConvFunctor (tf1/axqconv/axqconv.cc:113-278) for quint8 x quint8 -> qint32 with
+ * offset_output 0, mult 1, shift 0 (:354-356): the seven loops, the per-product zero-point correction (:228-247),
+ * taps outside the image reading the input offset (:213-216), the functor's own padding origin (:153-163).
+ * table is indexed [input_code * 256 + filter_code] (approximate_selector.h:101-103).  Pinned by brute force
+ * against the exact table (then it is the plain integer convolution of the offset-corrected codes).
+ * padding: AXO_PAD_SAME / AXO_PAD_VALID; output [batches][out_h][out_w][filter_count]. */
+void axo_axconv2d_tf1(const uint16_t *table, const uint8_t *input, int batches, int in_h, int in_w, int in_depth,
+                      int input_offset, const uint8_t *filter, int filter_h, int filter_w, int filter_count,
+                      int filter_offset, int stride, int padding, int32_t *output, int out_h, int out_w);
+
+/* AxTune column remap of ApproximateSelector::init (tf1/axqconv/approximate_selector.h:52-85). */
+void axo_table_tune_weights(const uint16_t *table, uint16_t *tuned);
 
 #ifdef __cplusplus
 }

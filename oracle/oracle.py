@@ -200,6 +200,32 @@ def lut_gemm_codes(table, a, b):
     return acc
 
 
+def axconv2d_tf1(table, input_codes, filter_codes, input_offset, filter_offset, stride=1, padding="SAME"):
+    """tf1 AxConv2D reference functor; output shape by TensorFlow's GetWindowedOutputSize."""
+    x = np.ascontiguousarray(input_codes, np.uint8)
+    f = np.ascontiguousarray(filter_codes, np.uint8)
+    table = np.ascontiguousarray(table, np.uint16)
+    n, h, w, c = x.shape
+    kh, kw, c2, co = f.shape
+    assert c == c2
+    if padding == "SAME":
+        oh, ow = -(-h // stride), -(-w // stride)
+    else:
+        oh, ow = (h - kh + stride) // stride, (w - kw + stride) // stride
+    out = np.zeros((n, oh, ow, co), np.int32)
+    lib().axo_axconv2d_tf1(_p(table, ctypes.c_uint16), _p(x, ctypes.c_uint8), n, h, w, c, int(input_offset),
+                           _p(f, ctypes.c_uint8), kh, kw, co, int(filter_offset), int(stride),
+                           1 if padding == "SAME" else 0, _p(out, ctypes.c_int32), oh, ow)
+    return out
+
+
+def table_tune_weights(table):
+    table = np.ascontiguousarray(table, np.uint16).reshape(-1)
+    tuned = np.zeros(65536, np.uint16)
+    lib().axo_table_tune_weights(_p(table, ctypes.c_uint16), _p(tuned, ctypes.c_uint16))
+    return tuned
+
+
 def time_reference_chunk(table, x, f, in_min, in_max, f_min, f_max, patches, strides=(1, 1), padding="SAME",
                          dilations=(1, 1)):
     """Seconds the reference-faithful single-thread path needs for the first `patches` output pixels."""

@@ -364,3 +364,32 @@ def test_fake_approx_conv2d_layer_all_zero_input(pkg):
     w = torch.from_numpy(np.random.default_rng(1).standard_normal((3, 3, 4, 8)).astype(np.float32)).to(dev)
     y = pkg.FakeApproxConv2D((1, 1), pkg.synth.table_exact(), "same")(x, w)
     assert torch.isfinite(y).all() and float(y.abs().max()) == 0.0
+
+
+AXCONV_TF1 = [
+    ((2, 9, 9, 8), (3, 3, 8, 12), 1, "SAME", (-1.0, 1.0, -0.5, 0.5)),
+    ((1, 10, 13, 5), (3, 3, 5, 7), 2, "SAME", (0.0, 6.0, -1.0, 1.0)),       # input zero point 0
+    ((1, 12, 12, 4), (5, 5, 4, 3), 3, "VALID", (-2.0, 1.0, -0.1, 0.3)),
+    ((1, 11, 11, 3), (3, 3, 3, 5), 4, "VALID", (-1.0, 1.0, -1.0, 1.0)),     # the functor's origin goes negative here
+    ((2, 7, 7, 256), (3, 3, 256, 16), 1, "SAME", (-1.0, 1.0, -0.5, 0.5)),   # K split over tiles
+]
+
+
+@pytest.mark.parametrize("case", AXCONV_TF1, ids=[str(i) for i in range(len(AXCONV_TF1))])
+def test_tf1_axconv2d_vs_reference_functor(pkg, oracle, case):
+    from tf_approximate_amd import ops
+    xs, fs, stride, padding, mm = case
+    rng = np.random.default_rng(xs[1] + fs[3])
+    x = rng.integers(0, 256, size=xs).astype(np.uint8)
+    f = rng.integers(0, 256, size=fs).astype(np.uint8)
+    table_np = ops.tune_table(pkg.synth.table_noisy(7))
+    assert np.array_equal(table_np, oracle.table_tune_weights(pkg.synth.table_noisy(7)))
+    table = pkg.TruthTable(table_np, 8)
+    dev = gpu_util.dev()
+    out, lo, hi = ops.ax_conv2d(torch.from_numpy(x).to(dev), torch.from_numpy(f).to(dev), *mm,
+                                [1, stride, stride, 1], padding, table)
+    off_in = ops.float_to_quantized_unclamped_quint8(0.0, mm[0], mm[1])
+    off_f = ops.float_to_quantized_unclamped_quint8(0.0, mm[2], mm[3])
+    want = oracle.axconv2d_tf1(table_np, x, f, off_in, off_f, stride, padding)
+    assert np.array_equal(out.cpu().numpy(), want)
+    assert lo < 0 < hi

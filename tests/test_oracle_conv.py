@@ -216,3 +216,55 @@ def test_committed_config1_vectors(oracle, pkg, golden_dir):
         assert np.array_equal(y, z["y_" + tname])
     # K = 144 fp32 terms in the epilogue: a few 1e-6 of the output maximum
     assert refimpl.linf_rel(z["y_exact"], refimpl.torch_conv2d_f64(z["x"], z["f"])) < 1e-5
+
+
+# ---- tf1 AxConv2D functor and AxTune ---------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [((2, 7, 6, 3), (3, 3, 3, 4), 1, "SAME"), ((1, 9, 9, 2), (3, 2, 2, 5), 2, "SAME"),
+                                   ((1, 8, 10, 3), (3, 3, 3, 2), 2, "VALID"), ((1, 5, 5, 1), (1, 1, 1, 3), 1, "VALID")])
+def test_tf1_axconv2d_exact_table_is_integer_convolution(oracle, shape):
+    """With t[a][b] = a*b every product term collapses to (a - offset_input) * (b - offset_filter), taps outside
+    the image contribute 0: the plain zero-padded integer convolution, computed here by a library routine."""
+    import torch
+    xs, fs, stride, padding = shape
+    rng = np.random.default_rng(sum(xs) + sum(fs))
+    x = rng.integers(0, 256, size=xs).astype(np.uint8)
+    f = rng.integers(0, 256, size=fs).astype(np.uint8)
+    off_in, off_f = 117, 131
+    got = oracle.axconv2d_tf1(oracle.table_exact(), x, f, off_in, off_f, stride, padding)
+    want = refimpl.torch_conv2d_f64(x.astype(np.float64) - off_in, f.astype(np.float64) - off_f, (stride, stride), padding)
+    assert got.shape == want.shape
+    assert np.array_equal(got.astype(np.int64), np.rint(want).astype(np.int64))
+
+
+def test_tf1_axconv2d_brute_force_with_noisy_table(oracle, pkg):
+    rng = np.random.default_rng(4)
+    x = rng.integers(0, 256, size=(1, 4, 5, 2)).astype(np.uint8)
+    f = rng.integers(0, 256, size=(3, 3, 2, 3)).astype(np.uint8)
+    table = pkg.synth.table_noisy(7).reshape(256, 256).astype(np.int64)
+    off_in, off_f = 3, 200
+    got = oracle.axconv2d_tf1(table.astype(np.uint16), x, f, off_in, off_f, 1, "SAME")
+    want = np.zeros((1, 4, 5, 3), np.int64)
+    for oy in range(4):
+        for ox in range(5):
+            for oc in range(3):
+                for fy in range(3):
+                    for fx in range(3):
+                        for ic in range(2):
+                            iy, ix = oy + fy - 1, ox + fx - 1
+                            a = int(x[0, iy, ix, ic]) if 0 <= iy < 4 and 0 <= ix < 5 else off_in
+                            b = int(f[fy, fx, ic, oc])
+                            want[0, oy, ox, oc] += table[a, b] - a * off_f - b * off_in + off_in * off_f
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+def test_tf1_table_tuning(oracle, pkg):
+    exact = oracle.table_exact()
+    assert np.array_equal(oracle.table_tune_weights(exact), np.asarray(exact).reshape(-1))  # nothing beats exact columns
+    noisy = pkg.synth.table_truncated(4).reshape(256, 256).astype(np.int64)
+    i = np.arange(256, dtype=np.int64)
+    err = np.abs(i[None, :, None] * i[:, None, None] - noisy[None, :, :]).sum(axis=1)   # err[w][w2]
+    tuned = oracle.table_tune_weights(noisy.astype(np.uint16)).reshape(256, 256)
+    for w in range(256):
+        best = err[w].min()
+        w2 = w if err[w][w] == best else int(np.argmax(err[w] == best))                 # ties: w itself, else the first
+        assert np.array_equal(tuned[:, w], noisy[:, w2]), w

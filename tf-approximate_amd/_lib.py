@@ -59,6 +59,8 @@ SYMBOLS = [
     ("axc_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_fake_approx_conv2d", ctypes.c_int, [_vp, _desc, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
+    ("axc_axconv2d_quint8", ctypes.c_int, [_vp, _desc, _vp, _vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp, _sz, _vp]),
+    ("axc_table_tune_weights", ctypes.c_int, [_vp, _vp]),
     ("axc_quantize", ctypes.c_int, [_vp, _i64, _f, _f, _vp, _vp]),
     ("axc_conv2d_minmax_acc_i32", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax_acc_i32", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),

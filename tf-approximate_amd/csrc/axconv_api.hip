@@ -2,9 +2,11 @@
 #include "axconv_internal.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <string>
@@ -47,7 +49,7 @@ struct ProfEntry {
     int64_t launches = 0;
 };
 std::mutex g_prof_mutex;
-bool g_prof_enabled = false;
+std::atomic<bool> g_prof_enabled{false};
 std::map<std::string, ProfEntry> g_prof;
 
 struct ProfScope {
@@ -55,12 +57,18 @@ struct ProfScope {
     hipStream_t stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     bool on;
-    ProfScope(const char *n, hipStream_t s) : name(n), stream(s), on(g_prof_enabled)
+    ProfScope(const char *n, hipStream_t s) : name(n), stream(s), on(g_prof_enabled.load())
     {
-        if (on && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess)
-            (void)hipEventRecord(e0, stream);
-        else
+        if (!on)
+            return;
+        if (hipEventCreate(&e0) != hipSuccess) {
             on = false;
+        } else if (hipEventCreate(&e1) != hipSuccess) {
+            (void)hipEventDestroy(e0);
+            on = false;
+        } else {
+            (void)hipEventRecord(e0, stream);
+        }
     }
     ~ProfScope()
     {
@@ -392,7 +400,7 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
               const uint8_t *input_codes, const uint8_t *filter_codes, int input_zero_code,
               float in_min, float in_max, float f_min, float f_max, float *out_f, int32_t *out_i,
               void *workspace, size_t workspace_bytes, void *stream_v, bool layer_mode = false,
-              const float *bias = nullptr, int activation = AXC_ACT_NONE)
+              const float *bias = nullptr, int activation = AXC_ACT_NONE, const int *pad_before_override = nullptr)
 {
     if (!table || !desc)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
@@ -404,6 +412,10 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         return rc;
     if (pd.empty)
         return AXC_OK;
+    if (pad_before_override) { // a caller with its own padding rule (tf1 AxConv2D); the plan does not depend on it
+        pd.g.ph = pad_before_override[0];
+        pd.g.pw = pad_before_override[1];
+    }
     const bool codes_mode = input_codes != nullptr;
     if ((!codes_mode && (!input || !filter)) || (codes_mode && !filter_codes) || (!out_f && !out_i))
         return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
@@ -691,6 +703,80 @@ int axc_fake_approx_conv2d(const axc_table *table, const axc_conv2d_desc *desc, 
         return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
     return run_dense(table, desc, input, filter, nullptr, nullptr, 0, 0.0f, 0.0f, 0.0f, 0.0f, output, nullptr, workspace,
                      workspace_bytes, stream, true, bias, activation);
+}
+
+// tf1 AxConv2D: filter origin offsets of ReferenceAxConvFunctor (tf1/axqconv/axqconv.cc:153-163), C integer division
+static void axconv_tf1_pads(const ConvGeom &g, int padding, int pads[2])
+{
+    const int extra = padding == AXC_PAD_VALID ? 1 : 0;
+    pads[0] = ((g.OH - 1) * g.sh + g.KH - g.H + extra) / 2;
+    pads[1] = ((g.OW - 1) * g.sw + g.KW - g.W + extra) / 2;
+}
+
+int axc_axconv2d_quint8(const axc_table *table, const axc_conv2d_desc *desc, const uint8_t *input,
+                        const uint8_t *filter, int32_t offset_input, int32_t offset_filter, int32_t *output,
+                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!desc)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    // AxQuantizedConv2DOp's attribute checks (tf1/axqconv/axqconv.cc:297-325)
+    if (desc->strides[1] != desc->strides[2])
+        return fail(AXC_INVALID_ARGUMENT, "Current implementation only supports equal length strides in the row and "
+                                          "column dimensions.");
+    if (desc->dilations[1] != 1 || desc->dilations[2] != 1)
+        return fail(AXC_INVALID_ARGUMENT, "Current implementation only supports dilated rate as 1 in the row and "
+                                          "column dimensions.");
+    if (desc->padding != AXC_PAD_SAME && desc->padding != AXC_PAD_VALID)
+        return fail(AXC_INVALID_ARGUMENT, "padding must be SAME or VALID");
+    if (offset_input < 0 || offset_input > 255) // the reference stores it in a quint8 for taps outside the image (:215)
+        return fail(AXC_INVALID_ARGUMENT, "offset_input must be in [0, 255]");
+    PreparedDense pd;
+    int rc = prepare_dense(desc, &pd);
+    if (rc != AXC_OK)
+        return rc;
+    if (pd.empty)
+        return AXC_OK;
+    if (!input || !filter || !output)
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    int pads[2];
+    axconv_tf1_pads(pd.g, desc->padding, pads);
+    rc = run_dense(table, desc, nullptr, nullptr, input, filter, offset_input, 0.0f, 0.0f, 0.0f, 0.0f, nullptr, output,
+                   workspace, workspace_bytes, stream, false, nullptr, AXC_ACT_NONE, pads);
+    if (rc != AXC_OK || pd.g.K == 0)
+        return rc;
+    pd.g.ph = pads[0];
+    pd.g.pw = pads[1];
+    char *ws = static_cast<char *>(workspace);
+    ProfScope ps("axconv_correction", static_cast<hipStream_t>(stream));
+    AXC_HIP(launch_axconv_correction(input, filter, pd.g, offset_input, offset_filter,
+                                     reinterpret_cast<int32_t *>(ws + pd.ws.psum_off),
+                                     reinterpret_cast<int32_t *>(ws + pd.ws.fsum_off), output,
+                                     static_cast<hipStream_t>(stream)));
+    return AXC_OK;
+}
+
+// AxTune of ApproximateSelector::init (tf1/axqconv/approximate_selector.h:52-85): every weight column w is replaced
+// by the column w2 whose products are closest (sum of absolute errors over all inputs) to the exact i * w.
+int axc_table_tune_weights(const uint16_t *table, uint16_t *tuned)
+{
+    if (!table || !tuned)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    std::vector<uint16_t> src(table, table + 65536); // table and tuned may alias
+    for (int w = 0; w < 256; ++w) {
+        int wpos = -1, werr = 0;
+        for (int w2 = 0; w2 < 256; ++w2) {
+            int sumerr = 0;
+            for (int i = 0; i < 256; ++i)
+                sumerr += abs(i * w - (int)src[i * 256 + w2]);
+            if (sumerr < werr || (werr == sumerr && w2 == w) || wpos < 0) {
+                werr = sumerr;
+                wpos = w2;
+            }
+        }
+        for (int i = 0; i < 256; ++i)
+            tuned[i * 256 + w] = src[i * 256 + wpos];
+    }
+    return AXC_OK;
 }
 
 int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6])

@@ -138,6 +138,8 @@ hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float i
 hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream);
 hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials, float *out_f, int32_t *out_i,
                                   hipStream_t stream);
+hipError_t launch_axconv_correction(const uint8_t *codes, const uint8_t *fcodes, const ConvGeom &g, int offset_input,
+                                    int offset_filter, int32_t *asum, int32_t *bsum, int32_t *out, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t stream);
 hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
                                    uint8_t *wcodes, float *fsum, hipStream_t stream);

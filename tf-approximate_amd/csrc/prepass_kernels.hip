@@ -559,6 +559,76 @@ hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *
     return hipGetLastError();
 }
 
+// ---- integer zero-point correction of the tf1 AxConv2D op (tf1/axqconv/axqconv.cc:228-247) ----
+// total = sum(T[a][b] - a*offset_filter - b*offset_input + offset_input*offset_filter) over the patch, where a tap
+// outside the image has a = offset_input.  The LUT-GEMM gives sum(T); these kernels give sum(a) per output pixel and
+// sum(b) per output column, and the last one combines them.
+__global__ void __launch_bounds__(256) code_patch_sums_kernel(const uint8_t *__restrict__ codes, ConvGeom g,
+                                                               int offset_input, int32_t *__restrict__ asum)
+{
+    const int64_t m = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= g.M)
+        return;
+    const int n = (int)(m / ((int64_t)g.OH * g.OW));
+    const int rem = (int)(m - (int64_t)n * g.OH * g.OW);
+    const int oh = rem / g.OW, ow = rem - oh * g.OW;
+    const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
+    int32_t s = 0;
+    for (int kh = 0; kh < g.KH; ++kh)
+        for (int kw = 0; kw < g.KW; ++kw) {
+            const int ih = ih0 + kh * g.dh, iw = iw0 + kw * g.dw;
+            if ((unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W) {
+                const uint8_t *src = codes + (((int64_t)n * g.H + ih) * g.W + iw) * g.C;
+                for (int c = 0; c < g.C; ++c)
+                    s += src[c];
+            } else {
+                s += offset_input * g.C;
+            }
+        }
+    asum[m] = s;
+}
+
+__global__ void __launch_bounds__(256) code_filter_sums_kernel(const uint8_t *__restrict__ fcodes, int K, int Co,
+                                                                int32_t *__restrict__ bsum)
+{
+    const int col = blockIdx.x * blockDim.x + threadIdx.x;
+    if (col >= Co)
+        return;
+    int32_t s = 0;
+    for (int k = 0; k < K; ++k)
+        s += fcodes[(int64_t)k * Co + col];
+    bsum[col] = s;
+}
+
+__global__ void __launch_bounds__(256) axconv_correct_kernel(int32_t *__restrict__ out, int64_t mc, int Co,
+                                                              const int32_t *__restrict__ asum,
+                                                              const int32_t *__restrict__ bsum, int offset_input,
+                                                              int offset_filter, int K)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= mc)
+        return;
+    const int64_t m = i / Co;
+    const int col = (int)(i - m * Co);
+    // wraps like the reference's int32 arithmetic would
+    const int64_t t = (int64_t)out[i] - (int64_t)asum[m] * offset_filter - (int64_t)bsum[col] * offset_input +
+                      (int64_t)K * offset_input * offset_filter;
+    out[i] = (int32_t)t;
+}
+
+hipError_t launch_axconv_correction(const uint8_t *codes, const uint8_t *fcodes, const ConvGeom &g, int offset_input,
+                                    int offset_filter, int32_t *asum, int32_t *bsum, int32_t *out, hipStream_t stream)
+{
+    hipLaunchKernelGGL(code_patch_sums_kernel, dim3(blocks_for(g.M, 256)), dim3(256), 0, stream, codes, g, offset_input,
+                       asum);
+    hipLaunchKernelGGL(code_filter_sums_kernel, dim3(blocks_for(g.Co, 256)), dim3(256), 0, stream, fcodes, g.K, g.Co,
+                       bsum);
+    const int64_t mc = g.M * g.Co;
+    hipLaunchKernelGGL(axconv_correct_kernel, dim3(blocks_for(mc, 256)), dim3(256), 0, stream, out, mc, g.Co, asum, bsum,
+                       offset_input, offset_filter, g.K);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t stream)
 {
     for (int64_t done = 0; done < n; done += (int64_t)1 << 30) { // int-sized pieces

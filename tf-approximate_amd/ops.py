@@ -7,6 +7,8 @@ stream); all arithmetic happens in libaxconv_hip.so.
 """
 import ctypes
 
+import numpy as np
+
 import torch
 
 from . import _lib
@@ -224,6 +226,69 @@ class FakeApproxConv2D:
                                               self.activation, out.data_ptr(), ws.data_ptr(), ws.numel(),
                                               _stream_ptr(inputs.device)))
         return out
+
+
+# ---- tf1 AxConv2D (tf1/axqconv/axqconv.cc) ----------------------------------------------------------------------
+def float_to_quantized_unclamped_quint8(value, range_min, range_max):
+    """TensorFlow's FloatToQuantizedUnclamped<quint8> (tensorflow/core/kernels/quantization_utils.h), which the
+    reference calls with value 0 to get the zero points (tf1/axqconv/axqconv.cc:350-353).  Restated from the
+    published algorithm; nothing in the reference pins it (third-party code)."""
+    if range_max == range_min:
+        return 0
+    steps = 256.0
+    range_adjust = steps / (steps - 1.0)
+    rng = (float(range_max) - float(range_min)) * range_adjust
+    scale = steps / rng
+
+    def rnd(v):  # std::round: half away from zero
+        return int(np.floor(abs(v) + 0.5)) * (1 if v >= 0 else -1)
+    return rnd(float(value) * scale) - rnd(float(range_min) * scale)
+
+
+def quantization_range_for_multiplication(min_a, max_a, min_b, max_b):
+    """TensorFlow's QuantizationRangeForMultiplication<quint8, quint8, qint32> (same header): the float range the
+    qint32 output of AxConv2D stands for (tf1/axqconv/axqconv.cc:427-431).  Third-party, restated."""
+    f32 = np.float32
+    a_one = f32((f32(max_a) - f32(min_a)) / f32(255.0))
+    b_one = f32((f32(max_b) - f32(min_b)) / f32(255.0))
+    c_one = f32(a_one * b_one)
+    return float(f32(c_one * f32(-2147483648.0))), float(f32(c_one * f32(2147483647.0)))
+
+
+def tune_table(table):
+    """AxTune of the tf1 op (tf1/axqconv/approximate_selector.h:52-85) applied to a uint16[65536] table."""
+    lib = _lib.load()
+    src = np.ascontiguousarray(table, np.uint16).reshape(-1)
+    if src.size != 65536:
+        raise InvalidArgumentError("table must hold 65536 entries")
+    out = np.zeros(65536, np.uint16)
+    _check(lib.axc_table_tune_weights(src.ctypes.data, out.ctypes.data))
+    return out
+
+
+def ax_conv2d(input, filter, min_input, max_input, min_filter, max_filter, strides, padding, table):
+    """The tf1 op AxConv2D (registration tf1/axqconv/axqconv.cc:66-94): quint8 codes in (uint8 tensors on the GPU),
+    (qint32 output, min_output, max_output) out.  `table` is a TruthTable (AxMult / AxTune already applied)."""
+    lib = _lib.load()
+    if input.dtype != torch.uint8 or filter.dtype != torch.uint8:
+        raise UnimplementedError("AxConv2D: only quint8 input and filter are registered")
+    if not input.is_cuda or not filter.is_cuda:
+        raise InvalidArgumentError("input and filter must be tensors on the GPU")
+    input, filter = input.contiguous(), filter.contiguous()
+    desc = make_desc(tuple(input.shape), tuple(filter.shape), list(strides), padding, (), "NHWC", (1, 1, 1, 1), 8)
+    dims = conv2d_geometry(desc)
+    nbytes = ctypes.c_size_t()
+    _check(lib.axc_conv2d_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+    ws = _workspace(input.device, nbytes.value)
+    out = torch.empty((dims.batch, int(dims.out_rows), int(dims.out_cols), dims.out_depth), dtype=torch.int32,
+                      device=input.device)
+    off_in = float_to_quantized_unclamped_quint8(0.0, min_input, max_input)
+    off_f = float_to_quantized_unclamped_quint8(0.0, min_filter, max_filter)
+    with torch.cuda.device(input.device):
+        _check(lib.axc_axconv2d_quint8(table.handle, ctypes.byref(desc), input.data_ptr(), filter.data_ptr(), off_in, off_f,
+                                       out.data_ptr(), ws.data_ptr(), ws.numel(), _stream_ptr(input.device)))
+    lo, hi = quantization_range_for_multiplication(min_input, max_input, min_filter, max_filter)
+    return out, lo, hi
 
 
 def conv2d_tile_plan(input_shape, filter_shape, strides=(1, 1, 1, 1), padding="SAME", dilations=(1, 1, 1, 1)):
