@@ -181,3 +181,24 @@ def test_missing_library_fails_loudly(pkg, monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libaxconv_hip.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _lib.load()
+
+
+def test_table_file_tool_round_trip_and_reference_format(pkg, golden_dir, tmp_path):
+    """tables.py writes the reference's file format: its exact table is byte-identical to the reference's
+    mul8u_1JFF.bin (the exact multiplier), and a written table reads back unchanged."""
+    import subprocess
+    import sys
+    from tf_approximate_amd import tables
+    out = tmp_path / "exact.bin"
+    tool = os.path.join(os.path.dirname(golden_dir), "..", "tf-approximate_amd", "tables.py")
+    r = subprocess.run([sys.executable, tool, "exact", str(out)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    with open(out, "rb") as a, open(os.path.join(golden_dir, "tables", "mul8u_1JFF.bin"), "rb") as b:
+        assert a.read() == b.read()
+    t = pkg.synth.table_noisy(3)
+    tables.write_table(tmp_path / "n.bin", t)
+    assert np.array_equal(tables.read_table(tmp_path / "n.bin"), np.asarray(t).reshape(-1))
+    stats = tables.error_stats(tables.read_table(out))
+    assert stats["wrong_entries"] == 0 and stats["symmetric"]
+    with pytest.raises(ValueError):
+        tables.write_table(tmp_path / "bad.bin", np.zeros(10))
