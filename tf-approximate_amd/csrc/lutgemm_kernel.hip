@@ -474,7 +474,15 @@ template <int NT, bool OUT_I32>
 static hipError_t launch_one(const DenseParams &p, hipStream_t stream)
 {
     auto kernel = lutgemm_expand_kernel<NT, OUT_I32>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+    // The generated assembly addresses LDS from offset 0: that holds as long as the kernel has no static LDS in
+    // front of its dynamic allocation.
+    hipFuncAttributes attr;
+    hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
+    if (e != hipSuccess)
+        return e;
+    if (attr.sharedSizeBytes != 0)
+        return hipErrorInvalidConfiguration;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kDenseLdsBytes + kDenseParkBytes);
     if (e != hipSuccess)
         return e;
