@@ -462,16 +462,17 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         AXC_HIP(launch_layer_quant(input, (int64_t)g.N * g.H * g.W * g.C, filter, (int64_t)g.K * g.Co, g.K, partials,
                                    lq_dev, stream));
     }
+    bool quantized_by_patch_sums = false;
+    if (out_f && !codes_mode) {
+        ProfScope ps("patch_sums", stream);
+        AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums));
+    }
     if (codes_mode) {
         ProfScope ps("codes_relayout", stream);
         AXC_HIP(launch_codes_relayout(input_codes, g, zp4, xq, stream));
-    } else {
+    } else if (!quantized_by_patch_sums) {
         ProfScope ps("quantize_relayout", stream);
         AXC_HIP(launch_quantize_relayout(input, g, tq_in, lq_dev, xq, nullptr, stream));
-    }
-    if (out_f && !codes_mode) {
-        ProfScope ps("patch_sums", stream);
-        AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream));
     }
     {
         ProfScope ps("filter_pack", stream);

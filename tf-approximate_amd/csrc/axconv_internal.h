@@ -123,11 +123,13 @@ __device__ inline uint32_t quantize_code(float v, float offset, float inv_scale)
 // ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
 hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
                                     uint32_t *xq, float *chsum, hipStream_t stream);
+// With xq_fused / fused given, 1x1 stride-1 layers also get their quantized activations from this pass
+// (*fused = true); the caller then skips launch_quantize_relayout.
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
-                             float *psum, hipStream_t stream);
+                             float *psum, hipStream_t stream, uint32_t *xq_fused = nullptr, bool *fused = nullptr);
 hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
                               float *partials, LayerQuant *lq_dev, hipStream_t stream);
-constexpr int kMinMaxBlocks = 512;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch
+constexpr int kMinMaxBlocks = 2048;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch
 hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
                                  hipStream_t stream);
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,

@@ -218,9 +218,14 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
 __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, ConvGeom g, int rb,
                                                                 int in_rows, const TensorQuant tq,
                                                                 const LayerQuant *__restrict__ lq_dev,
-                                                                float *__restrict__ psum)
+                                                                float *__restrict__ psum, uint32_t *__restrict__ xq)
 {
+    // xq != nullptr (1x1 filters, stride 1: every input row is copied by exactly one block): the block also
+    // quantizes what it copies, which saves the separate quantize pass over the input.
     const TensorQuant qt = lq_dev ? lq_dev->in : tq;
+    if (xq && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
+            xq[(int64_t)g.N * g.H * g.C4 * g.W + i] = qt.zp4;
     extern __shared__ __align__(16) unsigned char ps_lds[];
     float *const rows = reinterpret_cast<float *>(ps_lds);
     const int t = threadIdx.x;
@@ -241,6 +246,12 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
                 if (inb)
                     v = fake_quant_value4(*reinterpret_cast<const float4 *>(src + (int64_t)w * g.C), qt);
                 *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
+                if (xq && inb)
+                    xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + w] =
+                        phys_row(quantize_code(v.x, qt.offset, qt.inv_scale)) |
+                        (phys_row(quantize_code(v.y, qt.offset, qt.inv_scale)) << 8) |
+                        (phys_row(quantize_code(v.z, qt.offset, qt.inv_scale)) << 16) |
+                        (phys_row(quantize_code(v.w, qt.offset, qt.inv_scale)) << 24);
             }
         }
     } else {
@@ -449,13 +460,33 @@ __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t *__restrict__ ds
 // ---- the Keras layer's pre-step: per-tensor min / max and the quantization constants, all on the device ----
 // (tf2/python/keras/layers/fake_approx_convolutional.py:233-242: reduce_min / reduce_max of the batch and of
 // the kernel, then fake quantization with them.)  Stage 1: one (min, max) pair per workgroup.
-__global__ void __launch_bounds__(256) minmax_partial_kernel(const float *__restrict__ v, int64_t n,
+// The first blocks_a workgroups reduce tensor a, the others tensor b (one launch for the input and the filter).
+__global__ void __launch_bounds__(256) minmax_partial_kernel(const float *__restrict__ a, int64_t na, int blocks_a,
+                                                              const float *__restrict__ b, int64_t nb,
                                                               float *__restrict__ partials)
 {
     __shared__ float smin[256], smax[256];
+    const bool second = (int)blockIdx.x >= blocks_a;
+    const float *__restrict__ v = second ? b : a;
+    const int64_t n = second ? nb : na;
+    const int block = second ? (int)blockIdx.x - blocks_a : (int)blockIdx.x;
+    const int nblocks = second ? (int)gridDim.x - blocks_a : blocks_a;
+    partials += second ? 2 * kMinMaxBlocks : 0;
     float lo = INFINITY, hi = -INFINITY;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int64_t stride = (int64_t)nblocks * blockDim.x;
+    const int64_t tid = (int64_t)block * blockDim.x + threadIdx.x;
+    int64_t done = 0;
+    if (((uintptr_t)v & 15) == 0) { // 16 bytes per lane while they last, the remainder one float at a time
+        const float4 *v4 = reinterpret_cast<const float4 *>(v);
+        const int64_t n4 = n / 4;
+        for (int64_t i = tid; i < n4; i += stride) {
+            const float4 x = v4[i];
+            lo = fminf(fminf(lo, x.x), fminf(fminf(x.y, x.z), x.w));
+            hi = fmaxf(fmaxf(hi, x.x), fmaxf(fmaxf(x.y, x.z), x.w));
+        }
+        done = n4 * 4;
+    }
+    for (int64_t i = done + tid; i < n; i += stride) {
         const float x = v[i];
         lo = fminf(lo, x);
         hi = fmaxf(hi, x);
@@ -471,8 +502,8 @@ __global__ void __launch_bounds__(256) minmax_partial_kernel(const float *__rest
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        partials[2 * blockIdx.x] = smin[0];
-        partials[2 * blockIdx.x + 1] = smax[0];
+        partials[2 * block] = smin[0];
+        partials[2 * block + 1] = smax[0];
     }
 }
 
@@ -548,13 +579,12 @@ hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *
                               float *partials, LayerQuant *lq_dev, hipStream_t stream)
 {
     auto blocks = [](int64_t n) {
-        const int64_t b = (n + 256 * 16 - 1) / (256 * 16);
+        const int64_t b = (n + 256 * 32 - 1) / (256 * 32);
         return (int)(b < 1 ? 1 : (b > kMinMaxBlocks ? kMinMaxBlocks : b));
     };
     const int b_in = blocks(n_input), b_f = blocks(n_filter);
-    hipLaunchKernelGGL(minmax_partial_kernel, dim3(b_in), dim3(256), 0, stream, input, n_input, partials);
-    hipLaunchKernelGGL(minmax_partial_kernel, dim3(b_f), dim3(256), 0, stream, filter, n_filter,
-                       partials + 2 * kMinMaxBlocks);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(b_in + b_f), dim3(256), 0, stream, input, n_input, b_in, filter,
+                       n_filter, partials);
     hipLaunchKernelGGL(layer_quant_kernel, dim3(1), dim3(256), 0, stream, partials, b_in, b_f, K, lq_dev);
     return hipGetLastError();
 }
@@ -740,8 +770,10 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const Ten
 }
 
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
-                             float *psum, hipStream_t stream)
+                             float *psum, hipStream_t stream, uint32_t *xq_fused, bool *fused)
 {
+    if (fused)
+        *fused = false;
     const bool vec = (g.C & 3) == 0 && ((uintptr_t)x & 15) == 0;
     if (vec && g.OW <= 1024) {
         // largest band of output rows whose input rows fit in 96 KiB of LDS and whose pixels fit in one block,
@@ -760,6 +792,11 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
         if (rb > 0) {
             int threads = ((rb * g.OW + 63) / 64) * 64;
             threads = threads < 512 ? 512 : threads;   // the copy into LDS wants more threads than there are pixels
+            // 1x1, stride 1, no padding: bands partition the input rows, and the fast copy loop is in use
+            const bool fuse = xq_fused && fused && g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 &&
+                              g.pw == 0 && threads % g.C4 == 0;
+            if (fuse)
+                *fused = true;
             const size_t lds = (size_t)in_rows * row_bytes;
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(patch_sums_rows_kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
@@ -767,7 +804,7 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 return e;
             const int bands = (g.OH + rb - 1) / rb;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(g.N * bands)), dim3(threads), lds, stream, x, g,
-                               rb, in_rows, tq, lq_dev, psum);
+                               rb, in_rows, tq, lq_dev, psum, fuse ? xq_fused : nullptr);
             return hipGetLastError();
         }
     }
