@@ -1,0 +1,65 @@
+"""Seeded random layer shapes against the oracle: ragged channel / column counts, strides, dilations, both
+paddings, tiny and K-heavy layers, so that every tile-plan branch (column-tile widths, K splits, the ragged tail of
+the tile order, partial wavefront-rows) and every pre-pass variant meets odd sizes."""
+import numpy as np
+import pytest
+
+import gpu_util
+import refimpl
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_case(rng):
+    kh, kw = (int(v) for v in rng.choice([1, 1, 2, 3, 3, 5], size=2))
+    sh, sw = (int(v) for v in rng.choice([1, 1, 2, 3], size=2))
+    dh, dw = (int(v) for v in rng.choice([1, 1, 1, 2], size=2))
+    c = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 31, 32, 64, 100, 256]))
+    co = int(rng.choice([1, 2, 3, 4, 7, 8, 15, 16, 17, 30, 32, 33, 48, 64, 65, 100]))
+    n = int(rng.integers(1, 4))
+    h = int(rng.integers((kh - 1) * dh + 1, 24))
+    w = int(rng.integers((kw - 1) * dw + 1, 24))
+    if c >= 100:   # keep the oracle quick
+        h, w = min(h, 10), min(w, 10)
+    padding = str(rng.choice(["SAME", "VALID"]))
+    lo = float(rng.choice([-1.0, 0.0, -3.0]))
+    mm = (lo, lo + float(rng.choice([1.0, 2.5])), -0.5, 0.25)
+    return (n, h, w, c), (kh, kw, c, co), (sh, sw), (dh, dw), padding, mm
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_layer_vs_oracle(pkg, oracle, seed):
+    rng = np.random.default_rng(1000 + seed)
+    xs, fs, strides, dil, padding, mm = _random_case(rng)
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, mm, seed=seed)
+    table = pkg.synth.table_random(seed) if seed % 2 else pkg.synth.table_asymmetric()
+    y, acc = gpu_util.run_op(pkg, table, x, f, mm, strides, padding, dil)
+    rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding, dilations=dil)
+    assert rc == 0
+    assert acc.shape == acc_ref.shape, (xs, fs, strides, dil, padding)
+    assert np.array_equal(acc, acc_ref), (xs, fs, strides, dil, padding)
+    assert refimpl.linf_rel(y, y_ref) <= 1e-5, (xs, fs, strides, dil, padding)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_layer_entry_point_vs_composition(pkg, oracle, seed):
+    """The same for the layer entry point (off-grid inputs: the fused fake quantization has real work to do)."""
+    import torch
+    rng = np.random.default_rng(2000 + seed)
+    xs, fs, strides, dil, padding, mm = _random_case(rng)
+    x = rng.uniform(mm[0], mm[1], size=xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * 0.3).astype(np.float32)
+    bias = rng.uniform(-1, 1, size=fs[3]).astype(np.float32)
+    table = pkg.synth.table_noisy(seed)
+    dev = gpu_util.dev()
+    layer = pkg.FakeApproxConv2D(strides, table, padding, dilation_rate=dil, activation="relu" if seed % 2 else None)
+    y = layer(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev), torch.from_numpy(bias).to(dev)).cpu().numpy()
+    r = (float(x.min()), float(x.max()), float(w.min()), float(w.max()))
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    rc, y_ref, _ = oracle.conv2d_fast(table, fq(x, r[0], r[1]), fq(w, r[2], r[3]), *r, strides=strides, padding=padding,
+                                      dilations=dil)
+    assert rc == 0
+    y_ref = (y_ref + bias).astype(np.float32)
+    if seed % 2:
+        y_ref = np.maximum(y_ref, 0.0)
+    assert refimpl.linf_rel(y, y_ref) <= 1e-5, (xs, fs, strides, dil, padding)
