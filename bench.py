@@ -215,6 +215,17 @@ def main():
             "seconds": round(secs, 2),
             "gpu_vs_sample_linf": linf,
         }
+        # Not the reference's behaviour (its CPU op is single-threaded): the oracle's pre-quantized int32 loop with
+        # OpenMP over the output pixels on the host cores this process may use, on the first images of the batch.
+        cores = max(1, min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "64"))))
+        images = max(1, min(n, 16))
+        t_omp = time.perf_counter()
+        rc, _, _ = oracle.conv2d_fast(table, x[:images], f, *mm, strides=strides, padding="SAME", threads=cores)
+        t_omp = time.perf_counter() - t_omp
+        if rc == 0:
+            cpu["openmp_variant"] = {"value": round(images * oh * ow * co * taps_c / t_omp / 1e9, 3), "unit": "GMAC/s",
+                                     "cores": cores, "sample": "first %d images, int32 accumulate, filter quantized "
+                                     "once, OpenMP over output pixels" % images, "seconds": round(t_omp, 2)}
 
     result = {
         "metric": "approx_gmac_per_s",

@@ -180,8 +180,7 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
             const int ih = lih[i] + kh * g.dh, iw = liw[i] + kw * g.dw;
             v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (lbase[i] >= 0 && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W && c0 + j * 4 < g.C)
-                v[i] = fake_quant_value4(
-                    *reinterpret_cast<const float4 *>(x + ((int64_t)(lbase[i] + ih) * g.W + iw) * g.C + c0 + j * 4), qt);
+                v[i] = *reinterpret_cast<const float4 *>(x + ((int64_t)(lbase[i] + ih) * g.W + iw) * g.C + c0 + j * 4);
         }
     };
     float s = 0.0f;
@@ -189,8 +188,9 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
     for (int it = 0; it < iters; ++it) {
         __syncthreads(); // previous slice consumed
 #pragma unroll
-        for (int i = 0; i < kPsLoads; ++i)
-            *reinterpret_cast<float4 *>(&tile[(pl0 + i * (kPsTile / kQuads)) * kPsRow + j * 4]) = v[i];
+        for (int i = 0; i < kPsLoads; ++i)   // 0.0f (a tap outside the image) lies on the grid: snapping keeps it 0.0f
+            *reinterpret_cast<float4 *>(&tile[(pl0 + i * (kPsTile / kQuads)) * kPsRow + j * 4]) =
+                qt.fq ? fake_quant_value4(v[i], qt) : v[i];
         __syncthreads();
         if (it + 1 < iters)
             fetch(it + 1);
@@ -375,7 +375,12 @@ __device__ __forceinline__ void filter_sums_block(const int block, const float *
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
             const int k = k0 + rsub + i * (kFsThreads / 64);
-            v[i] = (k < K && col0 + cl < Co) ? fake_quant_value(filter[(int64_t)k * Co + col0 + cl], q) : 0.0f;
+            v[i] = (k < K && col0 + cl < Co) ? filter[(int64_t)k * Co + col0 + cl] : 0.0f;
+        }
+        if (q.fq) { // after the loads, so that they all stay in flight together
+#pragma unroll
+            for (int i = 0; i < kPer; ++i)
+                v[i] = fake_quant_value(v[i], q);   // padding zeros lie on the grid or are never summed
         }
         __syncthreads(); // previous pass consumed
 #pragma unroll
