@@ -543,7 +543,9 @@ int run_depthwise(const axc_table *table, const axc_conv2d_desc *desc, const flo
         return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     if (taps == 0) {
-        AXC_HIP(hipMemsetAsync(out_f ? (void *)out_f : (void *)out_i, 0, (size_t)M * C * 4, stream));
+        // a fill kernel rather than hipMemsetAsync: callers may capture the stream into a graph
+        AXC_HIP(launch_fill_u32(out_f ? reinterpret_cast<uint32_t *>(out_f) : reinterpret_cast<uint32_t *>(out_i), M * C, 0u,
+                                stream));
         return AXC_OK;
     }
     const size_t wcodes_bytes = align_up((size_t)taps * C);
