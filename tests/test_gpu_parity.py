@@ -393,3 +393,31 @@ def test_tf1_axconv2d_vs_reference_functor(pkg, oracle, case):
     want = oracle.axconv2d_tf1(table_np, x, f, off_in, off_f, stride, padding)
     assert np.array_equal(out.cpu().numpy(), want)
     assert lo < 0 < hi
+
+
+def test_hip_graph_capture_and_replays(pkg):
+    """The op and the layer entry point allocate nothing and record no memset nodes: a captured graph of a small
+    network replays to the eager result every time, with eager work and synchronisation between the replays."""
+    from tf_approximate_amd import networks
+    table = pkg.synth.table_noisy(7)
+    shape = (4, 16, 16, 3)
+    x = torch.from_numpy(np.random.default_rng(9).uniform(0, 1, size=shape).astype(np.float32)).to(gpu_util.dev())
+    for fused in (False, True):
+        net = networks.ApproxNetwork(networks.cifar_resnet_program(blocks_per_stage=1), shape, table, seed=4,
+                                     fused_layers=fused)
+        eager, _ = net.forward(x, calibrate=True)
+        eager = eager.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            net.forward(x)                      # warm-up on the capture stream: workspaces grow here, not in the graph
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out, _ = net.forward(x)
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+            out.zero_()                         # eager work between the replays; also proves the replay rewrites it
+            torch.cuda.synchronize()
