@@ -83,8 +83,24 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
 
     const uint32_t zero_off = quantize_code(0.0f, p.in_offset, p.in_inv_scale) * 2u;
     const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;   // (output row segment, channel), channel fastest
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t item = (int64_t)blockIdx.x * blockDim.x + tid; item < items; item += stride) {
+    // Neighbouring output rows read the same input rows.  Workgroups go to the 8 XCDs round-robin and every XCD
+    // has its own L2, so each XCD gets one contiguous band of output rows (whole rows): an input row is then
+    // fetched from memory by one L2 instead of by up to three.
+    const int64_t per_row = (int64_t)nseg * p.C;
+    const int64_t rows_total = (int64_t)p.N * p.OH;
+    int64_t first = 0, last = items, stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t start = (int64_t)blockIdx.x * blockDim.x + tid;
+    if ((gridDim.x & 7) == 0) {
+        const int xcd = blockIdx.x & 7;
+        const int64_t rows_per_xcd = (rows_total + 7) / 8;
+        first = rows_per_xcd * xcd * per_row;
+        last = rows_per_xcd * (xcd + 1) * per_row;
+        last = last < items ? last : items;
+        stride = (int64_t)(gridDim.x >> 3) * blockDim.x;
+        start = first + (int64_t)(blockIdx.x >> 3) * blockDim.x + tid;
+    }
+    (void)first;
+    for (int64_t item = start; item < last; item += stride) {
         const int c = (int)(item % p.C);
         const int64_t rs = item / p.C;
         const int seg = (int)(rs % nseg);
@@ -223,7 +239,9 @@ hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hi
             (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;
         const int64_t blocks = (items + kBlockThreads - 1) / kBlockThreads;
-        const int g3 = (int)(blocks < cus ? blocks : cus);
+        int g3 = (int)(blocks < cus ? blocks : cus);
+        if (g3 >= 64)
+            g3 &= ~7;   // a multiple of 8 workgroups: the kernel then keeps bands of output rows on one XCD each
         if (p.sw == 1)
             return out_i32 ? launch_with_table_lds(depthwise_lut3x3_kernel<1, true>, g3, stream, p, seg_len, nseg)
                            : launch_with_table_lds(depthwise_lut3x3_kernel<1, false>, g3, stream, p, seg_len, nseg);
