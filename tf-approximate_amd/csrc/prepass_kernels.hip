@@ -220,8 +220,9 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
                                                                 const LayerQuant *__restrict__ lq_dev,
                                                                 float *__restrict__ psum, uint32_t *__restrict__ xq)
 {
-    // xq != nullptr (1x1 filters, stride 1: every input row is copied by exactly one block): the block also
-    // quantizes what it copies, which saves the separate quantize pass over the input.
+    // xq != nullptr: the block also quantizes the input rows it owns among those it copies (the rows under its
+    // own band of output rows; the launcher has checked that these lie inside every block's window and together
+    // cover the image), which saves the separate quantize pass over the input.
     const TensorQuant qt = lq_dev ? lq_dev->in : tq;
     if (xq && blockIdx.x == 0)
         for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
@@ -230,28 +231,47 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
     float *const rows = reinterpret_cast<float *>(ps_lds);
     const int t = threadIdx.x;
     const int bands = (g.OH + rb - 1) / rb;
-    const int n = blockIdx.x / bands;
-    const int oh0 = (blockIdx.x - n * bands) * rb;
+    // consecutive bands (which share input rows) go to the same XCD: blocks are dealt round-robin over 8 XCDs
+    const int per_xcd = gridDim.x / 8, extra = gridDim.x % 8, xcd = blockIdx.x & 7;
+    const int bid = xcd * per_xcd + (xcd < extra ? xcd : extra) + (blockIdx.x >> 3);
+    const int n = bid / bands;
+    const int oh0 = (bid - n * bands) * rb;
     const int ih_first = oh0 * g.sh - g.ph;  // input row held in LDS row 0 (may lie outside the image)
+    const int own_lo = oh0 * g.sh;           // owned input rows: [own_lo, own_hi)
+    const int own_hi = (oh0 + rb >= g.OH) ? g.H : (oh0 + rb) * g.sh;
     const int pitch = g.C + 4;
     if (blockDim.x % g.C4 == 0) {
-        // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns
+        // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns, four
+        // 16-byte loads in flight at a time
         const int q = t % g.C4, w0 = t / g.C4, wstep = blockDim.x / g.C4;
-        for (int r = 0; r < in_rows; ++r) {
-            const int ih = ih_first + r;
-            const bool inb = (unsigned)ih < (unsigned)g.H;
-            const float *src = x + (((int64_t)n * g.H + (inb ? ih : 0)) * g.W) * g.C + q * 4;
-            for (int w = w0; w < g.W; w += wstep) {
-                float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                if (inb)
-                    v = fake_quant_value4(*reinterpret_cast<const float4 *>(src + (int64_t)w * g.C), qt);
-                *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
-                if (xq && inb)
-                    xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + w] =
-                        phys_row(quantize_code(v.x, qt.offset, qt.inv_scale)) |
-                        (phys_row(quantize_code(v.y, qt.offset, qt.inv_scale)) << 8) |
-                        (phys_row(quantize_code(v.z, qt.offset, qt.inv_scale)) << 16) |
-                        (phys_row(quantize_code(v.w, qt.offset, qt.inv_scale)) << 24);
+        const int wsteps = (g.W + wstep - 1) / wstep;
+        const int iters = in_rows * wsteps;
+        for (int it0 = 0; it0 < iters; it0 += 4) {
+            float4 v[4];
+            int rr[4], ww[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int it = it0 + u;
+                rr[u] = it / wsteps;
+                ww[u] = w0 + (it - rr[u] * wsteps) * wstep;
+                const int ih = ih_first + rr[u];
+                v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (it < iters && ww[u] < g.W && (unsigned)ih < (unsigned)g.H)
+                    v[u] = *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + ww[u]) * g.C + q * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (it0 + u >= iters || ww[u] >= g.W)
+                    continue;
+                const int ih = ih_first + rr[u];
+                const float4 f = fake_quant_value4(v[u], qt);   // rows outside the image stay zero
+                *reinterpret_cast<float4 *>(&rows[(rr[u] * g.W + ww[u]) * pitch + q * 4]) = f;
+                if (xq && (unsigned)ih < (unsigned)g.H && ih >= own_lo && ih < own_hi)
+                    xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + ww[u]] =
+                        phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
+                        (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
+                        (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
+                        (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
             }
         }
     } else {
@@ -797,9 +817,11 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
         if (rb > 0) {
             int threads = ((rb * g.OW + 63) / 64) * 64;
             threads = threads < 512 ? 512 : threads;   // the copy into LDS wants more threads than there are pixels
-            // 1x1, stride 1, no padding: bands partition the input rows, and the fast copy loop is in use
-            const bool fuse = xq_fused && fused && g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 &&
-                              g.pw == 0 && threads % g.C4 == 0;
+            // Band b owns input rows [b*rb*sh, (b+1)*rb*sh), the last band up to H.  They are quantized by the
+            // block that holds them if every band's window (rows b*rb*sh - ph onwards, in_rows of them) contains
+            // its owned rows, the last window reaches the last image row, and the fast copy loop is in use.
+            const bool fuse = xq_fused && fused && g.sh - 1 + g.ph <= (g.KH - 1) * g.dh &&
+                              (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0;
             if (fuse)
                 *fused = true;
             const size_t lds = (size_t)in_rows * row_bytes;
