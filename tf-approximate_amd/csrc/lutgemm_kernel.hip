@@ -204,13 +204,6 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             park[(2 * r + 1) * kDenseThreads] = rvalid[r] ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
         }
 
-        int32_t acc[R][NT];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-                acc[r][j] = 0;
-
         const uint32_t wq_tile = ((uint32_t)ct * (uint32_t)fills_all + (uint32_t)f0) * 128u; // this tile's first codes
         const int fills_left = fills_all - f0;              // codes may be prefetched past the split, not past the end
 
@@ -299,19 +292,32 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         uint32_t codes[4];
         tap_setup();
         load_acts(actA);
-        load_codes(0, codes);
-        load_rows(codes, rows);       // fill 0
-        load_codes(1, codes);
-        __syncthreads();              // the previous tile's last phase is done with every buffer
-        store_stage(rows, 0);
-        load_rows(codes, rows);       // fill 1
-        load_codes(2, codes);
+        {
+            // two rounds of loads, each in flight together: the filter codes of fills 0-3, then the table rows
+            // of fills 0-2 (the accumulators are not live yet, so the registers are there)
+            uint32_t codes0[4], codes1[4], codes2[4];
+            u32x4 rows0[4], rows1[4];
+            load_codes(0, codes0);
+            load_codes(1, codes1);
+            load_codes(2, codes2);
+            load_codes(3, codes);
+            load_rows(codes0, rows0);
+            load_rows(codes1, rows1);
+            load_rows(codes2, rows);
+            __syncthreads();          // the previous tile's last phase and epilogue are done with every buffer
+            store_stage(rows0, 0);
+            store_stage(rows1, 1);
+        }
         __syncthreads();
         derive(0);
-        store_stage(rows, 1);
-        load_rows(codes, rows);       // fill 2
-        load_codes(3, codes);
         __syncthreads();
+
+        int32_t acc[R][NT];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+                acc[r][j] = 0;
 
         // One phase per fill, one barrier per phase.
         PhaseConsts k;
@@ -367,50 +373,68 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             return p.relu ? fmaxf(v, 0.0f) : v;
         };
         constexpr bool kTransposed = NT <= 32;
+        // Every global load of the epilogue is issued here, ahead of the first store: loads and stores complete in
+        // issue order, so a load behind a store would wait until that store has reached memory.
+        float ps[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t m = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64 + lane;
+            ps[r] = (!OUT_I32 && rvalid[r]) ? p.psum[m] : 0.0f;
+        }
         if (kTransposed && (g.Co & 3) == 0) {
             constexpr int Q = NT / 4;                 // 16-byte quads (lanes) per pixel
             constexpr int PITCH = NT * 4 + 16;        // bytes per pixel in LDS: the +16 spreads pixels over the banks
             unsigned char *const wl = lds + (size_t)wave * 64 * PITCH;
             typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+            // Behind the transposition a lane stores the same four columns of every pixel it handles: the terms
+            // that depend on the column (filter sum, bias) are applied there, from four registers each.
+            const int quad = lane % Q, colq = ct * NT + quad * 4;
+            float t3q[4], biasq[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = colq + j < g.Co ? colq + j : g.Co - 1;
+                t3q[j] = OUT_I32 ? 0.0f : __fmul_rn(e_m1, p.fsum[c]);
+                biasq[j] = (!OUT_I32 && p.bias) ? p.bias[c] : 0.0f;
+            }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (r >= (int)nr_s)
                     break;
                 const int64_t m0 = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
                 const int nvalid = (int)(row_end - m0 < 64 ? row_end - m0 : 64);
-                const float psum = (!OUT_I32 && lane < nvalid) ? p.psum[m0 + lane] : 0.0f;
-                const float t1 = __fmul_rn(e_m2, psum);
+                const float t1 = __fmul_rn(e_m2, ps[r]);
 #pragma unroll
                 for (int set = 0; set < SETS; ++set) {
                     const int h = (c0 + set) & (SETS - 1);
                     uint32_t w[8];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        if (OUT_I32) {
+                        if (OUT_I32)
                             w[e] = (uint32_t)acc[r][set * 8 + e];
-                        } else {
-                            int col = ct * NT + h * 8 + e;
-                            col = col < g.Co ? col : g.Co - 1;
-                            const float t0 = __fmul_rn((float)acc[r][set * 8 + e], e_s1xs2);
-                            const float t2 = __fadd_rn(t0, t1);
-                            const float t3 = __fmul_rn(e_m1, p.fsum[col]);
-                            const float t4 = __fadd_rn(t2, t3);
-                            w[e] = __float_as_uint(finish(__fsub_rn(t4, e_km), col));
-                        }
+                        else
+                            w[e] = __float_as_uint(__fadd_rn(__fmul_rn((float)acc[r][set * 8 + e], e_s1xs2), t1));
                     }
                     u32x4s lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
                     *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32) = lo;
                     *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32 + 16) = hi;
                 }
-                const int quad = lane % Q, col = ct * NT + quad * 4;
                 uint32_t *const out = OUT_I32 ? reinterpret_cast<uint32_t *>(p.out_i) + (int64_t)ksi * g.M * g.Co
                                               : reinterpret_cast<uint32_t *>(p.out_f);
 #pragma unroll
                 for (int i = 0; i < Q; ++i) {
                     const int pix = i * (64 / Q) + lane / Q;
-                    const u32x4s d = *reinterpret_cast<const u32x4s *>(wl + pix * PITCH + quad * 16);
-                    if (pix < nvalid && col < g.Co)
-                        *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + col) = d;
+                    u32x4s d = *reinterpret_cast<const u32x4s *>(wl + pix * PITCH + quad * 16);
+                    if (!OUT_I32) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            float v = __fsub_rn(__fadd_rn(__uint_as_float(d[j]), t3q[j]), e_km);
+                            if (p.bias)
+                                v = __fadd_rn(v, biasq[j]);
+                            d[j] = __float_as_uint(p.relu ? fmaxf(v, 0.0f) : v);
+                        }
+                    }
+                    if (pix < nvalid && colq < g.Co)
+                        *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq) = d;
                 }
             }
             continue;
@@ -421,8 +445,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 continue;
             const int64_t m = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64 + lane;
             // patch sum of the raw input in the reference's order (tap-major, channels ascending)
-            const float psum = OUT_I32 ? 0.0f : p.psum[m];
-            const float t1 = __fmul_rn(e_m2, psum);
+            const float t1 = __fmul_rn(e_m2, ps[r]);
 #pragma unroll
             for (int set = 0; set < SETS; ++set) {
                 const int h = (c0 + set) & (SETS - 1);
