@@ -12,8 +12,10 @@ barriers.  The macro interleaves, in one instruction stream with hand-counted s_
             code.  The LDS address of step s is ONE v_perm_b32 (byte 1 <- activation code: the rows of the two
             buffers interleave, 256 bytes apart; byte 0 <- the lane's chunk offset).  The reads run through a
             rolling window of eight that does not drain between pixels.  Each arrived chunk is accumulated
-            with eight v_add_u32_sdwa, one VALU op per table entry, the 16-bit halves being picked by the SDWA
-            source selector.  Step s accumulates into column group s % (NT / 8).
+            with eight VALU adds, one per table entry: the entry in the high half of a dword through the SDWA
+            source selector, the one in the low half by adding the whole dword (the surplus, 65536 times the
+            high entries, is subtracted once behind the last phase).  Step s accumulates into column group
+            s % (NT / 8).
   stage     the table rows of fill p+2 (in ROWS since the previous phase) go to staged-row buffer BUF.
   loads     table rows of fill p+3 -> ROWS (addresses from CODES), filter codes of fill p+4 -> CODES,
             activations of fill p+1 -> ANEXT; waited for at the end of the macro.
@@ -104,8 +106,14 @@ def emit(nt, buf):
         g = step % sets
         for e in range(8):
             c = "%%[c%d_%d]" % (r, g * 8 + e)
-            st.ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:%s"
-                   % (c, c, b + e // 2, "WORD_0" if e % 2 == 0 else "WORD_1"))
+            if e % 2 == 0:
+                # the whole dword: the accumulator of the even column collects lo + 65536 * hi (mod 2^32); the
+                # kernel takes 65536 * (sum of hi) off again behind the last phase.  A plain add issues at twice
+                # the rate of an SDWA one.
+                st.ins("v_add_u32 %s, %s, v%d" % (c, c, b + e // 2))
+            else:
+                st.ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
+                       % (c, c, b + e // 2))
 
     def prime(st):
         src = rotate(st, 0)

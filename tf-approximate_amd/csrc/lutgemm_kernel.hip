@@ -193,9 +193,16 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             const int64_t m = wrow + lane;
             rvalid[r] = m < row_end && wrow < wr_end;
             const int64_t mm = rvalid[r] ? m : row0;
-            const int n = (int)(mm / ((int64_t)g.OH * g.OW));
-            const int rem = (int)(mm - (int64_t)n * g.OH * g.OW);
-            const int oh = rem / g.OW;
+            int n, rem;
+            if (g.M <= 0x7fffffff) { // the usual case: 32-bit divisions (a 64-bit one costs several times more)
+                const uint32_t ohow = (uint32_t)(g.OH * g.OW);
+                n = (int)((uint32_t)mm / ohow);
+                rem = (int)((uint32_t)mm - (uint32_t)n * ohow);
+            } else {
+                n = (int)(mm / ((int64_t)g.OH * g.OW));
+                rem = (int)(mm - (int64_t)n * g.OH * g.OW);
+            }
+            const int oh = (int)((uint32_t)rem / (uint32_t)g.OW);
             const int ow = rem - oh * g.OW;
             const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
             // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
@@ -359,6 +366,14 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 phase(pcur + 1, actB, actA, std::integral_constant<int, 1>());
         }
 
+        // The phases add whole dwords (two 16-bit table entries) into the accumulator of the even column and the
+        // high entry alone into that of the odd column: even = sum(lo) + 65536 * sum(hi) modulo 2^32.
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < NT; j += 2)
+                acc[r][j] = (int32_t)((uint32_t)acc[r][j] - ((uint32_t)acc[r][j + 1] << 16));
+
         // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----
         // A lane holds NT consecutive columns of its pixel: stored as they are, one instruction would touch 64
         // different 64-byte pieces of memory.  The wavefront therefore turns each of its wavefront-rows
@@ -433,8 +448,14 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                             d[j] = __float_as_uint(p.relu ? fmaxf(v, 0.0f) : v);
                         }
                     }
-                    if (pix < nvalid && colq < g.Co)
-                        *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq) = d;
+                    if (pix < nvalid && colq < g.Co) {
+                        // the float output is not read again by this op: streamed past the caches, which keeps
+                        // them for the activations; split-K partial sums are read back at once and stay cached
+                        if (OUT_I32)
+                            *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq) = d;
+                        else
+                            __builtin_nontemporal_store(d, reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq));
+                    }
                 }
             }
             continue;
