@@ -180,6 +180,11 @@ int axc_profile_read(int index, char *name, size_t name_bytes, double *total_ms,
  * ceiling of the LDS-lookup roofline. */
 int axc_lds_gather_peak(double *lookups_per_second, void *stream);
 
+/* Conflict-free streaming ds_read_b128 rate of this GPU (bytes per second over all CUs): the ceiling of the
+ * LDS read port for 16-byte accesses, the width the LUT-GEMM reads its expanded table rows with.  A lookup
+ * moves at least its 2-byte table entry through that port. */
+int axc_lds_read_peak(double *bytes_per_second, void *stream);
+
 /* Properties of the current device the planner uses. */
 int axc_device_info(int *compute_units, int *lds_bytes_per_workgroup, int *clock_khz);
 

@@ -70,6 +70,7 @@ SYMBOLS = [
     ("axc_profile_read", ctypes.c_int, [ctypes.c_int, ctypes.c_char_p, _sz, ctypes.POINTER(ctypes.c_double),
                                         ctypes.POINTER(_i64)]),
     ("axc_lds_gather_peak", ctypes.c_int, [ctypes.POINTER(ctypes.c_double), _vp]),
+    ("axc_lds_read_peak", ctypes.c_int, [ctypes.POINTER(ctypes.c_double), _vp]),
     ("axc_device_info", ctypes.c_int, [ctypes.POINTER(ctypes.c_int)] * 3),
 ]
 

@@ -462,10 +462,12 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         AXC_HIP(launch_layer_quant(input, (int64_t)g.N * g.H * g.W * g.C, filter, (int64_t)g.K * g.Co, g.K, partials,
                                    lq_dev, stream));
     }
-    bool quantized_by_patch_sums = false;
+    bool quantized_by_patch_sums = false, filter_done = false;
     if (out_f && !codes_mode) {
-        ProfScope ps("patch_sums", stream);
-        AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums));
+        ProfScope ps("patch_sums", stream);   // carries the filter pre-pass along when it can
+        const FilterJob job = {filter, filter_codes, &pd.plan, tq_f, wq, fsum};
+        AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, &job,
+                                  &filter_done));
     }
     if (codes_mode) {
         ProfScope ps("codes_relayout", stream);
@@ -474,7 +476,7 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         ProfScope ps("quantize_relayout", stream);
         AXC_HIP(launch_quantize_relayout(input, g, tq_in, lq_dev, xq, nullptr, stream));
     }
-    {
+    if (!filter_done) {
         ProfScope ps("filter_pack", stream);
         AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, g, pd.plan, tq_f, lq_dev, wq,
                                    (out_f && !codes_mode) ? fsum : nullptr, stream));
@@ -917,7 +919,16 @@ int axc_lds_gather_peak(double *lookups_per_second, void *stream)
     if (!lookups_per_second)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
     *lookups_per_second = 0.0;
-    AXC_HIP(run_lds_gather_peak(lookups_per_second, static_cast<hipStream_t>(stream)));
+    AXC_HIP(run_lds_gather_peak(lookups_per_second, static_cast<hipStream_t>(stream), false));
+    return AXC_OK;
+}
+
+int axc_lds_read_peak(double *bytes_per_second, void *stream)
+{
+    if (!bytes_per_second)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    *bytes_per_second = 0.0;
+    AXC_HIP(run_lds_gather_peak(bytes_per_second, static_cast<hipStream_t>(stream), true));
     return AXC_OK;
 }
 

@@ -125,8 +125,20 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const Ten
                                     uint32_t *xq, float *chsum, hipStream_t stream);
 // With xq_fused / fused given, 1x1 stride-1 layers also get their quantized activations from this pass
 // (*fused = true); the caller then skips launch_quantize_relayout.
+// The filter pre-pass of the same layer (what launch_filter_pack would do), for a launch that can take it along.
+struct FilterJob {
+    const float *filter;
+    const uint8_t *filter_codes;
+    const DensePlan *plan;
+    TensorQuant tq;
+    uint16_t *wq;
+    float *fsum;
+};
+// xq_fused / fused: the launch may also quantize the input into xq (then *fused is set);
+// filter_job / filter_done: it may also do the filter pre-pass (then *filter_done is set).
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
-                             float *psum, hipStream_t stream, uint32_t *xq_fused = nullptr, bool *fused = nullptr);
+                             float *psum, hipStream_t stream, uint32_t *xq_fused = nullptr, bool *fused = nullptr,
+                             const FilterJob *filter_job = nullptr, bool *filter_done = nullptr);
 hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
                               float *partials, LayerQuant *lq_dev, hipStream_t stream);
 constexpr int kMinMaxBlocks = 2048;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch
@@ -146,6 +158,6 @@ hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t
 hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
                                    uint8_t *wcodes, float *fsum, hipStream_t stream);
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream);
-hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream);
+hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128);
 
 } // namespace axc

@@ -279,7 +279,32 @@ __global__ void __launch_bounds__(kBlockThreads) lds_gather_probe_kernel(uint32_
     out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;
 }
 
-hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream)
+// Streaming ds_read_b128: every lane reads its own 16 bytes of a contiguous 1 KiB per wavefront, no bank
+// conflicts.  The byte rate is the ceiling of the LDS read port for the access width the LUT-GEMM uses.
+__global__ void __launch_bounds__(kBlockThreads) lds_stream_probe_kernel(uint32_t *out, int iters)
+{
+    uint32_t *l32 = reinterpret_cast<uint32_t *>(lds_dw);
+    for (int i = threadIdx.x; i < kTableBytes / 4; i += blockDim.x)
+        l32[i] = (uint32_t)i * 2654435761u;
+    __syncthreads();
+    // a wavefront walks 8 x 1 KiB per iteration inside its own 16 KiB window
+    const uint32_t base = (uint32_t)(threadIdx.x & 63) * 16u + ((uint32_t)(threadIdx.x >> 6) & 7u) * 16384u;
+    uint32_t acc = 0;
+    for (int it = 0; it < iters; ++it) {
+        u32x4 v[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v[r]) : "v"(base), "n"(r * 1024));
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            acc += v[r].x ^ v[r].w;
+    }
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+
+hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128)
 {
     int dev = 0, cus = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -289,25 +314,27 @@ hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream)
     uint32_t *out = nullptr;
     e = hipMalloc(&out, (size_t)cus * kBlockThreads * sizeof(uint32_t));
     if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(lds_gather_probe_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kTableBytes);
+    auto probe = stream_b128 ? lds_stream_probe_kernel : lds_gather_probe_kernel;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(probe), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kTableBytes);
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (e == hipSuccess) e = hipEventCreate(&e0);
     if (e == hipSuccess) e = hipEventCreate(&e1);
     const int iters = 8000;
     if (e == hipSuccess) {
-        hipLaunchKernelGGL(lds_gather_probe_kernel, dim3(cus), dim3(kBlockThreads), kTableBytes, stream, out, 100);
+        hipLaunchKernelGGL(probe, dim3(cus), dim3(kBlockThreads), kTableBytes, stream, out, 100);
         e = hipEventRecord(e0, stream);
     }
     if (e == hipSuccess) {
-        hipLaunchKernelGGL(lds_gather_probe_kernel, dim3(cus), dim3(kBlockThreads), kTableBytes, stream, out, iters);
+        hipLaunchKernelGGL(probe, dim3(cus), dim3(kBlockThreads), kTableBytes, stream, out, iters);
         e = hipEventRecord(e1, stream);
     }
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     float ms = 0.0f;
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
     if (e == hipSuccess && ms > 0.0f)
-        *lookups_per_second = (double)cus * kBlockThreads * (double)iters * 16.0 / (ms * 1e-3);
+        // gather mode: 16 two-byte lookups per lane and iteration; stream mode: 8 x 16 bytes (the result is bytes/s)
+        *lookups_per_second = (double)cus * kBlockThreads * (double)iters * (stream_b128 ? 128.0 : 16.0) / (ms * 1e-3);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     (void)hipFree(out);

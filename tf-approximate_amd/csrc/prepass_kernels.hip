@@ -215,16 +215,19 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
 // pixel) and first copies the input rows they touch into LDS, so every input float is fetched from memory
 // about once (plus the halo) instead of once per filter tap; the sequential chains then read LDS only.
 // Pixels are padded to C + 4 floats so that the 16-byte reads of neighbouring threads fall into different banks.
-__global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, ConvGeom g, int rb,
-                                                                int in_rows, const TensorQuant tq,
-                                                                const LayerQuant *__restrict__ lq_dev,
-                                                                float *__restrict__ psum, uint32_t *__restrict__ xq)
+// bid / nblocks: index of this workgroup among those that do this work (in dispatch order, so that bid & 7 is
+// the XCD); nthreads: the threads of the workgroup that take part (the others only meet the barrier).
+__device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x, const ConvGeom &g, const int rb,
+                                                     const int in_rows, const TensorQuant &tq,
+                                                     const LayerQuant *__restrict__ lq_dev, float *__restrict__ psum,
+                                                     uint32_t *__restrict__ xq, const int bid_in, const int nblocks,
+                                                     const int nthreads)
 {
     // xq != nullptr: the block also quantizes the input rows it owns among those it copies (the rows under its
     // own band of output rows; the launcher has checked that these lie inside every block's window and together
     // cover the image), which saves the separate quantize pass over the input.
     const TensorQuant qt = lq_dev ? lq_dev->in : tq;
-    if (xq && blockIdx.x == 0)
+    if (xq && bid_in == 0)
         for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
             xq[(int64_t)g.N * g.H * g.C4 * g.W + i] = qt.zp4;
     extern __shared__ __align__(16) unsigned char ps_lds[];
@@ -232,18 +235,20 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
     const int t = threadIdx.x;
     const int bands = (g.OH + rb - 1) / rb;
     // consecutive bands (which share input rows) go to the same XCD: blocks are dealt round-robin over 8 XCDs
-    const int per_xcd = gridDim.x / 8, extra = gridDim.x % 8, xcd = blockIdx.x & 7;
-    const int bid = xcd * per_xcd + (xcd < extra ? xcd : extra) + (blockIdx.x >> 3);
+    const int per_xcd = nblocks / 8, extra = nblocks % 8, xcd = bid_in & 7;
+    const int bid = xcd * per_xcd + (xcd < extra ? xcd : extra) + (bid_in >> 3);
     const int n = bid / bands;
     const int oh0 = (bid - n * bands) * rb;
     const int ih_first = oh0 * g.sh - g.ph;  // input row held in LDS row 0 (may lie outside the image)
     const int own_lo = oh0 * g.sh;           // owned input rows: [own_lo, own_hi)
     const int own_hi = (oh0 + rb >= g.OH) ? g.H : (oh0 + rb) * g.sh;
     const int pitch = g.C + 4;
-    if (blockDim.x % g.C4 == 0) {
+    if (t >= nthreads) {
+        // not taking part in the copy
+    } else if (nthreads % g.C4 == 0) {
         // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns, four
         // 16-byte loads in flight at a time
-        const int q = t % g.C4, w0 = t / g.C4, wstep = blockDim.x / g.C4;
+        const int q = t % g.C4, w0 = t / g.C4, wstep = nthreads / g.C4;
         const int wsteps = (g.W + wstep - 1) / wstep;
         const int iters = in_rows * wsteps;
         for (int it0 = 0; it0 < iters; it0 += 4) {
@@ -277,7 +282,7 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
     } else {
         const int quads_per_row = g.W * g.C4;
         const int total = in_rows * quads_per_row;
-        for (int i = t; i < total; i += blockDim.x) {
+        for (int i = t; i < total; i += nthreads) {
             const int r = i / quads_per_row, rem = i - r * quads_per_row;
             const int w = rem / g.C4, q = rem - w * g.C4;
             const int ih = ih_first + r;
@@ -373,28 +378,29 @@ __device__ __forceinline__ void filter_pack_element(const int64_t i, const float
 
 // Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one thread per output column,
 // rows (h, w, c) ascending.
-// A block owns 64 columns; all 1024 threads stage up to 512 filter rows at a time into LDS (coalesced, every
+// A block owns 64 columns; all its threads (512 or 1024) stage up to 256 filter rows at a time into LDS (coalesced, every
 // load of a pass in flight at once), then the first 64 threads extend their column's sequential sum from LDS,
 // 32 independent LDS reads ahead of the dependent chain of adds.
-constexpr int kFsRows = 512, kFsThreads = 1024;
+constexpr int kFsRows = 256, kFsThreads = 1024; // 65 KiB of LDS: a launch that also does patch sums keeps their LDS size
 constexpr int kFsLdsBytes = kFsRows * 65 * 4;
 
 extern __shared__ __align__(16) unsigned char fs_lds[];
 
+template <int THREADS>
 __device__ __forceinline__ void filter_sums_block(const int block, const float *__restrict__ filter, int K, int Co,
                                                   const TensorQuant &q, float *__restrict__ fsum)
 {
-    constexpr int kBatch = 32, kPer = kFsRows * 64 / kFsThreads; // loads per thread per pass
+    constexpr int kBatch = 32, kPer = kFsRows * 64 / THREADS; // loads per thread per pass
     float *const stage = reinterpret_cast<float *>(fs_lds);
     const int col0 = block * 64;
     const int t = threadIdx.x;
-    const int cl = t & 63, rsub = t >> 6; // 16 rows per step
+    const int cl = t & 63, rsub = t >> 6; // THREADS / 64 rows per step
     float s = 0.0f;
     for (int k0 = 0; k0 < K; k0 += kFsRows) {
         float v[kPer];
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
-            const int k = k0 + rsub + i * (kFsThreads / 64);
+            const int k = k0 + rsub + i * (THREADS / 64);
             v[i] = (k < K && col0 + cl < Co) ? filter[(int64_t)k * Co + col0 + cl] : 0.0f;
         }
         if (q.fq) { // after the loads, so that they all stay in flight together
@@ -405,7 +411,7 @@ __device__ __forceinline__ void filter_sums_block(const int block, const float *
         __syncthreads(); // previous pass consumed
 #pragma unroll
         for (int i = 0; i < kPer; ++i)
-            stage[(rsub + i * (kFsThreads / 64)) * 65 + cl] = v[i];
+            stage[(rsub + i * (THREADS / 64)) * 65 + cl] = v[i];
         __syncthreads();
         if (t < 64) {
             const int nr = (K - k0 < kFsRows) ? K - k0 : kFsRows;
@@ -439,11 +445,51 @@ __global__ void __launch_bounds__(kFsThreads) filter_prep_kernel(const float *__
 {
     const TensorQuant q = lq_dev ? lq_dev->flt : tq;
     if ((int)blockIdx.x < sum_blocks) {
-        filter_sums_block((int)blockIdx.x, filter, taps * C, Co, q, fsum);
+        filter_sums_block<kFsThreads>((int)blockIdx.x, filter, taps * C, Co, q, fsum);
         return;
     }
     const int64_t i = (int64_t)(blockIdx.x - sum_blocks) * blockDim.x + threadIdx.x;
     filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, q, wq);
+}
+
+// The filter pre-pass of a layer is independent of its input pre-pass: as two launches they would run one after
+// the other, so the launch below carries both.  The first filter_blocks8 workgroups (a multiple of 8, which keeps
+// workgroup index mod 8 = XCD for the others) do the filter work of filter_prep_kernel, the rest the patch sums.
+struct FilterWork {
+    const float *filter;
+    const uint8_t *filter_codes;
+    int taps, C, C4, Co, nt, n_col_tiles;
+    TensorQuant tq;
+    uint16_t *wq;
+    int sum_blocks;
+    float *fsum;
+    int blocks;    // sum_blocks + pack blocks; 0: no filter work in this launch
+    int blocks8;   // blocks rounded up to a multiple of 8
+};
+
+__global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, const ConvGeom g, int rb,
+                                                                int in_rows, int nthreads, const TensorQuant tq,
+                                                                const LayerQuant *__restrict__ lq_dev,
+                                                                float *__restrict__ psum, uint32_t *__restrict__ xq,
+                                                                const FilterWork fw)
+{
+    if ((int)blockIdx.x < fw.blocks8) {
+        if ((int)blockIdx.x >= fw.blocks)
+            return;
+        const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
+        if ((int)blockIdx.x < fw.sum_blocks) { // the launcher gives these workgroups 512 or 1024 threads
+            if (blockDim.x == 512)
+                filter_sums_block<512>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
+            else
+                filter_sums_block<1024>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
+            return;
+        }
+        const int64_t i = (int64_t)((int)blockIdx.x - fw.sum_blocks) * blockDim.x + threadIdx.x;
+        filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+        return;
+    }
+    patch_sums_rows_body(x, g, rb, in_rows, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
+                         (int)gridDim.x - fw.blocks8, nthreads);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -795,10 +841,13 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const Ten
 }
 
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
-                             float *psum, hipStream_t stream, uint32_t *xq_fused, bool *fused)
+                             float *psum, hipStream_t stream, uint32_t *xq_fused, bool *fused,
+                             const FilterJob *filter_job, bool *filter_done)
 {
     if (fused)
         *fused = false;
+    if (filter_done)
+        *filter_done = false;
     const bool vec = (g.C & 3) == 0 && ((uintptr_t)x & 15) == 0;
     if (vec && g.OW <= 1024) {
         // largest band of output rows whose input rows fit in 96 KiB of LDS and whose pixels fit in one block,
@@ -824,14 +873,40 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                               (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0;
             if (fuse)
                 *fused = true;
-            const size_t lds = (size_t)in_rows * row_bytes;
+            size_t lds = (size_t)in_rows * row_bytes;
+            const int bands = (g.OH + rb - 1) / rb;
+            // the filter pre-pass rides along in the same launch (its workgroups want 512 or 1024 threads, so
+            // every workgroup gets that many; only `threads` of them take part in the patch sums)
+            FilterWork fw = {};
+            int block_threads = threads;
+            if (filter_job && filter_done) {
+                const DensePlan &plan = *filter_job->plan;
+                const int64_t total = (int64_t)plan.n_col_tiles * plan.fills * 64;
+                fw.filter = filter_job->filter;
+                fw.filter_codes = filter_job->filter_codes;
+                fw.taps = g.KH * g.KW;
+                fw.C = g.C;
+                fw.C4 = g.C4;
+                fw.Co = g.Co;
+                fw.nt = plan.nt;
+                fw.n_col_tiles = plan.n_col_tiles;
+                fw.tq = filter_job->tq;
+                fw.wq = filter_job->wq;
+                fw.sum_blocks = (filter_job->fsum && filter_job->filter) ? (int)blocks_for(g.Co, 64) : 0;
+                fw.fsum = filter_job->fsum;
+                block_threads = threads <= 512 ? 512 : 1024;
+                fw.blocks = fw.sum_blocks + (int)blocks_for(total, block_threads);
+                fw.blocks8 = (fw.blocks + 7) & ~7;
+                if (fw.sum_blocks && lds < (size_t)kFsLdsBytes)
+                    lds = kFsLdsBytes;
+                *filter_done = true;
+            }
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(patch_sums_rows_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kFsLdsBytes);
             if (e != hipSuccess)
                 return e;
-            const int bands = (g.OH + rb - 1) / rb;
-            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(g.N * bands)), dim3(threads), lds, stream, x, g,
-                               rb, in_rows, tq, lq_dev, psum, fuse ? xq_fused : nullptr);
+            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + g.N * bands)), dim3(block_threads),
+                               lds, stream, x, g, rb, in_rows, threads, tq, lq_dev, psum, fuse ? xq_fused : nullptr, fw);
             return hipGetLastError();
         }
     }

@@ -399,6 +399,13 @@ def lds_gather_peak():
     return v.value
 
 
+def lds_read_peak():
+    """Streaming ds_read_b128 rate in bytes/s over all CUs (measured)."""
+    v = ctypes.c_double()
+    _check(_lib.load().axc_lds_read_peak(ctypes.byref(v), None))
+    return v.value
+
+
 def device_info():
     a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     _check(_lib.load().axc_device_info(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
