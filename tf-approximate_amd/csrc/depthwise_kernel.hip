@@ -64,9 +64,17 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut_kernel(const Dept
 
 // 3x3 filters, dilation 1, column stride SW in {1, 2}: a thread owns one channel of a run of consecutive output
 // pixels of one output row and slides the 3x3 window along it.  Every input value is loaded and quantized once
-// per window row instead of once per tap, the nine filter codes of the channel live in registers as table row
-// offsets, and no 64-bit index arithmetic is left in the loop.  Same results as depthwise_lut_kernel: taps in
-// (kh, kw) order, zeros (code = zero point) outside the image.
+// per window row instead of once per tap, and the nine filter codes of the channel live in registers as table row
+// offsets.  Loads and stores go through buffer descriptors with 32-bit offsets: a column or row outside the image
+// gets an offset past the end of the buffer and reads 0.0f without a branch, and 0.0f quantizes to the zero-point
+// code, which is what a tap outside the image looks up.  Same results as depthwise_lut_kernel: taps in (kh, kw)
+// order, zeros (code = zero point) outside the image.
+typedef __amdgpu_buffer_rsrc_t dw_rsrc_t;
+__device__ __forceinline__ dw_rsrc_t dw_make_rsrc(const void *base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
 template <int SW, bool OUT_I32>
 __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const DepthwiseParams p, const int seg_len,
                                                                           const int nseg)
@@ -81,93 +89,101 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
     }
     __syncthreads();
 
-    const uint32_t zero_off = quantize_code(0.0f, p.in_offset, p.in_inv_scale) * 2u;
+    // the launcher has checked that input and output are below 2 GiB, so offsets from 0x70000000 up are outside
+    constexpr uint32_t kOutside = 0x70000000u;
+    const uint32_t x_bytes = (uint32_t)((int64_t)p.N * p.H * p.W * p.C * 4);
+    const uint32_t o_bytes = (uint32_t)(p.M * p.C * 4);
+    const dw_rsrc_t x_rsrc = dw_make_rsrc(p.x, x_bytes);
+    const dw_rsrc_t o_rsrc = dw_make_rsrc(OUT_I32 ? static_cast<const void *>(p.out_i) : static_cast<const void *>(p.out_f), o_bytes);
+    const uint32_t col_bytes = (uint32_t)p.C * 4u;           // bytes between neighbouring pixels of a row
+
     const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;   // (output row segment, channel), channel fastest
     // Neighbouring output rows read the same input rows.  Workgroups go to the 8 XCDs round-robin and every XCD
     // has its own L2, so each XCD gets one contiguous band of output rows (whole rows): an input row is then
     // fetched from memory by one L2 instead of by up to three.
     const int64_t per_row = (int64_t)nseg * p.C;
     const int64_t rows_total = (int64_t)p.N * p.OH;
-    int64_t first = 0, last = items, stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t last = items, stride = (int64_t)gridDim.x * blockDim.x;
     int64_t start = (int64_t)blockIdx.x * blockDim.x + tid;
     if ((gridDim.x & 7) == 0) {
         const int xcd = blockIdx.x & 7;
         const int64_t rows_per_xcd = (rows_total + 7) / 8;
-        first = rows_per_xcd * xcd * per_row;
+        const int64_t first = rows_per_xcd * xcd * per_row;
         last = rows_per_xcd * (xcd + 1) * per_row;
         last = last < items ? last : items;
         stride = (int64_t)(gridDim.x >> 3) * blockDim.x;
         start = first + (int64_t)(blockIdx.x >> 3) * blockDim.x + tid;
     }
-    (void)first;
+    constexpr int U = 4;                 // outputs per group
+    constexpr int NEW = U * SW;          // columns that enter the window per group
+    constexpr int CARRY = 3 - SW;        // columns the next group shares with this one
     for (int64_t item = start; item < last; item += stride) {
-        const int c = (int)(item % p.C);
-        const int64_t rs = item / p.C;
-        const int seg = (int)(rs % nseg);
-        const int64_t row = rs / nseg;                         // n * OH + oh
-        const int oh = (int)(row % p.OH);
-        const int n = (int)(row / p.OH);
+        // items < 2^31 here (the output is below 2 GiB): 32-bit divisions, a fraction of the cost of 64-bit ones
+        const uint32_t it32 = (uint32_t)item;
+        const uint32_t rs = it32 / (uint32_t)p.C;
+        const int c = (int)(it32 - rs * (uint32_t)p.C);
+        const uint32_t row = rs / (uint32_t)nseg;              // n * OH + oh
+        const int seg = (int)(rs - row * (uint32_t)nseg);
+        const int n = (int)(row / (uint32_t)p.OH);
+        const int oh = (int)(row - (uint32_t)n * (uint32_t)p.OH);
         const int ow0 = seg * seg_len;
-        const int ow1 = ow0 + seg_len < p.OW ? ow0 + seg_len : p.OW;
+        const int len = (ow0 + seg_len < p.OW ? ow0 + seg_len : p.OW) - ow0;
         const int ih0 = oh * p.sh - p.ph;
 
         uint32_t wrow[9];                                      // byte offset of the table row of each tap's filter code
 #pragma unroll
         for (int t = 0; t < 9; ++t)
             wrow[t] = (uint32_t)p.wcodes[t * p.C + c] * 512u;
-        const float fs = OUT_I32 ? 0.0f : p.fsum[c];
-        const float *rowp[3];
-        bool rowok[3];
+        const float t3 = OUT_I32 ? 0.0f : __fmul_rn(p.m1, p.fsum[c]);
+        uint32_t rowbase[3];                                   // byte offset of (n, ih, 0, c); outside for a row that is
 #pragma unroll
         for (int kh = 0; kh < 3; ++kh) {
             const int ih = ih0 + kh;
-            rowok[kh] = (unsigned)ih < (unsigned)p.H;
-            rowp[kh] = p.x + ((int64_t)n * p.H + (rowok[kh] ? ih : 0)) * p.W * p.C + c;
+            rowbase[kh] = (unsigned)ih < (unsigned)p.H
+                              ? (uint32_t)((((int64_t)n * p.H + ih) * p.W * p.C + c) * 4)
+                              : 0x80000000u;
         }
-        float val[3][3];
-        uint32_t off[3][3];                                    // activation code * 2 = byte offset inside a table row
-        auto fetch = [&](int kh, int iw, float &v, uint32_t &o) {
-            v = 0.0f;
-            o = zero_off;
-            if (rowok[kh] && (unsigned)iw < (unsigned)p.W) {
-                v = rowp[kh][iw * p.C];
-                o = quantize_code(v, p.in_offset, p.in_inv_scale) * 2u;
+        const int iw0 = ow0 * SW - p.pw;                       // input column under tap kw = 0 of the first output
+        auto col_off = [&](int iw) {                           // byte offset of column iw inside a row; outside if none
+            return (unsigned)iw < (unsigned)p.W ? (uint32_t)iw * col_bytes : kOutside;
+        };
+        auto load = [&](int kh, uint32_t coff) {
+            return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(rowbase[kh] + coff), 0, 0));
+        };
+        float cv[3][CARRY + NEW];                              // window columns of the group: values ...
+        uint32_t ca[3][CARRY + NEW];                           // ... and activation codes * 2 (byte offset in a table row)
+#pragma unroll
+        for (int t = 0; t < CARRY; ++t) {
+            const uint32_t coff = col_off(iw0 + t);
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh) {
+                cv[kh][t] = load(kh, coff);
+                ca[kh][t] = quantize_code(cv[kh][t], p.in_offset, p.in_inv_scale) * 2u;
+            }
+        }
+        // the columns that enter the window with the next group are loaded one group ahead
+        float pf[3][NEW];
+        auto prefetch = [&](int jfirst) {                      // new columns of outputs jfirst .. jfirst + U - 1
+#pragma unroll
+            for (int t = 0; t < NEW; ++t) {
+                const uint32_t coff = col_off(iw0 + jfirst * SW + CARRY + t);
+#pragma unroll
+                for (int kh = 0; kh < 3; ++kh)
+                    pf[kh][t] = load(kh, coff);
             }
         };
-        const int iw0 = ow0 * SW - p.pw;                       // input column under tap kw = 0 of the first output
-#pragma unroll
-        for (int kh = 0; kh < 3; ++kh)
-#pragma unroll
-            for (int kw = 0; kw < 3; ++kw)
-                fetch(kh, iw0 + kw, val[kh][kw], off[kh][kw]);
-        // The columns that enter the window for the next U outputs are loaded one group ahead, so that a thread
-        // keeps 3 * U * SW loads in flight instead of waiting for each output's own.
-        constexpr int U = 4, NC = U * SW;
-        const int len = ow1 - ow0;
-        float pf[3][NC];
-        auto prefetch = [&](int jfirst) {                       // new columns of outputs jfirst .. jfirst + U - 1
-#pragma unroll
-            for (int kh = 0; kh < 3; ++kh)
-#pragma unroll
-                for (int t = 0; t < NC; ++t) {
-                    const int j = jfirst + t / SW;               // the output this column first serves
-                    const int iw = iw0 + jfirst * SW + (3 - SW) + t;
-                    pf[kh][t] = 0.0f;
-                    if (j < len && rowok[kh] && (unsigned)iw < (unsigned)p.W)
-                        pf[kh][t] = rowp[kh][iw * p.C];
-                }
-        };
-        prefetch(1);
-        int64_t o_idx = ((int64_t)row * p.OW + ow0) * p.C + c;
+        prefetch(0);
+        uint32_t o_off = (uint32_t)((((int64_t)row * p.OW + ow0) * p.C + c) * 4);
         for (int j0 = 0; j0 < len; j0 += U) {
-            float cur[3][NC];
 #pragma unroll
             for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
-                for (int t = 0; t < NC; ++t)
-                    cur[kh][t] = pf[kh][t];
-            if (j0 + U + 1 < len + U)                            // something left to fetch for the next group
-                prefetch(j0 + U + 1);
+                for (int t = 0; t < NEW; ++t) {
+                    cv[kh][CARRY + t] = pf[kh][t];
+                    ca[kh][CARRY + t] = quantize_code(pf[kh][t], p.in_offset, p.in_inv_scale) * 2u;
+                }
+            if (j0 + U < len)
+                prefetch(j0 + U);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (j0 + u >= len)
@@ -178,39 +194,30 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                 for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
                     for (int kw = 0; kw < 3; ++kw) {
-                        psum = __fadd_rn(psum, val[kh][kw]);
-                        acc += (int32_t)*reinterpret_cast<const uint16_t *>(lds_dw + wrow[kh * 3 + kw] + off[kh][kw]);
+                        psum = __fadd_rn(psum, cv[kh][u * SW + kw]);
+                        acc += (int32_t)*reinterpret_cast<const uint16_t *>(lds_dw + wrow[kh * 3 + kw] + ca[kh][u * SW + kw]);
                     }
+                uint32_t outw;
                 if (OUT_I32) {
-                    p.out_i[o_idx] = acc;
+                    outw = (uint32_t)acc;
                 } else {
                     const float t0 = __fmul_rn((float)acc, p.s1xs2);
                     const float t1 = __fmul_rn(p.m2, psum);
                     const float t2 = __fadd_rn(t0, t1);
-                    const float t3 = __fmul_rn(p.m1, fs);
                     const float t4 = __fadd_rn(t2, t3);
-                    p.out_f[o_idx] = __fsub_rn(t4, p.k_m1xm2);
+                    outw = __float_as_uint(__fsub_rn(t4, p.k_m1xm2));
                 }
-                o_idx += p.C;
-                // slide the window to output j0 + u + 1: its new columns are cur[.][u*SW .. u*SW + SW - 1]
-                const int iw_new = iw0 + (j0 + u + 1) * SW + (3 - SW);
-#pragma unroll
-                for (int kh = 0; kh < 3; ++kh) {
-#pragma unroll
-                    for (int kw = 0; kw + SW < 3; ++kw) {
-                        val[kh][kw] = val[kh][kw + SW];
-                        off[kh][kw] = off[kh][kw + SW];
-                    }
-#pragma unroll
-                    for (int t = 0; t < SW; ++t) {
-                        const int kw = 3 - SW + t;
-                        const float v = cur[kh][u * SW + t];
-                        const bool inb = rowok[kh] && (unsigned)(iw_new + t) < (unsigned)p.W;
-                        val[kh][kw] = v;
-                        off[kh][kw] = inb ? quantize_code(v, p.in_offset, p.in_inv_scale) * 2u : zero_off;
-                    }
-                }
+                __builtin_amdgcn_raw_buffer_store_b32(outw, o_rsrc, (int)o_off, 0, 2); // nt: streamed past the caches, which
+                                                                                    // the input rows three output rows share need
+                o_off += col_bytes;
             }
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+                for (int t = 0; t < CARRY; ++t) {
+                    cv[kh][t] = cv[kh][NEW + t];
+                    ca[kh][t] = ca[kh][NEW + t];
+                }
         }
     }
 }
@@ -228,11 +235,14 @@ static hipError_t launch_with_table_lds(Kernel kernel, int grid, hipStream_t str
 
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream)
 {
+    // the sliding kernel addresses input and output with 32-bit byte offsets and keeps the top of that range free
     const bool sliding = p.KH == 3 && p.KW == 3 && p.dh == 1 && p.dw == 1 && (p.sw == 1 || p.sw == 2) &&
-                         (int64_t)p.W * p.C < (1ll << 31) / 4;
+                         (int64_t)p.N * p.H * p.W * p.C * 4 < 0x70000000ll && p.M * p.C * 4 < 0x70000000ll;
     if (sliding) {
-        // runs of at most 32 output pixels per thread: enough items to balance the CUs, few window restarts
-        const int nseg = (p.OW + 31) / 32;
+        // runs of at most 32 (stride 2: 16) output pixels per thread: enough items to balance the CUs, few window
+        // restarts, and the rows in flight on an XCD at one time still fit its L2
+        const int run = p.sw == 1 ? 32 : 16;
+        const int nseg = (p.OW + run - 1) / run;
         const int seg_len = (p.OW + nseg - 1) / nseg;
         int dev = 0, cus = 256;
         if (hipGetDevice(&dev) == hipSuccess)
