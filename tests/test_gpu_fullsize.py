@@ -117,3 +117,28 @@ def test_stress_layers_sampled_pixels(pkg, oracle, name, tname):
     table = pkg.synth.table_random(13) if tname == "random" else pkg.synth.table_exact()
     y, acc = gpu_util.run_op(pkg, table, x, f, MM, strides)
     _sampled_rows_check(pkg, oracle, table, x, f, MM, strides, acc, y, n_samples=24, seed=2)
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_depthwise_benchmark_shape_vs_oracle(pkg, oracle, stride):
+    """The depthwise benchmark layer's geometry (3x3 over 112x112x192, both strides) at batch 4, whole output against
+    the oracle: the runs of 32 / 16 output pixels per thread, the image borders and all three channel groups."""
+    xs, fs = (4, 112, 112, 192), (3, 3, 192, 1)
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=31 + stride)
+    x = x + np.float32(0.0017)          # off the quantization grid: patch sums differ from the dequantized codes
+    table = pkg.synth.table_random(17)
+    y, acc = gpu_util.run_op(pkg, table, x, f, MM, (stride, stride), depthwise=True)
+    rc, y_ref, acc_ref = oracle.depthwise_conv2d(table, x, f, *MM, strides=(stride, stride), padding="SAME",
+                                                  dilations=(1, 1))
+    assert rc == 0
+    assert np.array_equal(acc, acc_ref)
+    assert np.max(np.abs(y - y_ref)) <= 1e-5 * max(np.max(np.abs(y_ref)), 1e-30)
+
+
+def test_lds_probes_report_plausible_rates(pkg):
+    """The two measured ceilings of the bench line: the per-entry gather rate and the streaming 16-byte read rate.
+    A 16-byte read moves 8 entries, so the read port in entries/s must come out well above the gather rate."""
+    gather = pkg.ops.lds_gather_peak()
+    port = pkg.ops.lds_read_peak()
+    assert 1e12 < gather < 1e14
+    assert port / 2.0 > 2.0 * gather
