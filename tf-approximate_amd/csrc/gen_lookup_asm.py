@@ -108,8 +108,8 @@ def emit(nt, buf):
             c = "%%[c%d_%d]" % (r, g * 8 + e)
             if e % 2 == 0:
                 # the whole dword: the accumulator of the even column collects lo + 65536 * hi (mod 2^32); the
-                # kernel takes 65536 * (sum of hi) off again behind the last phase.  A plain add issues at twice
-                # the rate of an SDWA one.
+                # kernel takes 65536 * (sum of hi) off again behind the last phase.  One plain add instead of an
+                # SDWA one.
                 st.ins("v_add_u32 %s, %s, v%d" % (c, c, b + e // 2))
             else:
                 st.ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
