@@ -421,3 +421,63 @@ def test_hip_graph_capture_and_replays(pkg):
             assert torch.equal(out, eager)
             out.zero_()                         # eager work between the replays; also proves the replay rewrites it
             torch.cuda.synchronize()
+
+
+def test_concurrent_host_threads_through_the_c_abi(pkg, oracle):
+    """Two host threads drive the C ABI at the same time: one table, but a stream, a workspace and an output per
+    thread (what the header promises to support).  Each thread alternates two layer shapes for a few hundred calls;
+    every result must equal the one the same call gives alone."""
+    import ctypes
+    import threading
+    from tf_approximate_amd import _lib, ops
+    lib = _lib.load()
+    table = ops.TruthTable(pkg.synth.table_random(23), 8)
+    dev = gpu_util.dev()
+    shapes = [((2, 24, 24, 16), (3, 3, 16, 32), (1, 1, 1, 1)), ((1, 17, 19, 8), (1, 1, 8, 48), (1, 2, 2, 1)),
+              ((2, 15, 15, 12), (5, 5, 12, 20), (1, 1, 1, 1)), ((1, 30, 30, 4), (3, 3, 4, 70), (1, 2, 2, 1))]
+    jobs = []
+    for i, (xs, fs, st) in enumerate(shapes):
+        x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=40 + i)
+        desc = ops.make_desc(xs, fs, st, "SAME")
+        dims = _lib.ConvDims()
+        assert lib.axc_conv2d_geometry(ctypes.byref(desc), ctypes.byref(dims)) == 0
+        nbytes = ctypes.c_size_t()
+        assert lib.axc_conv2d_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0
+        xd, fd = torch.from_numpy(x).to(dev), torch.from_numpy(f).to(dev)
+        out_shape = (xs[0], int(dims.out_rows), int(dims.out_cols), fs[3])
+        ws = torch.empty(max(nbytes.value, 256), dtype=torch.uint8, device=dev)
+        y = torch.empty(out_shape, dtype=torch.float32, device=dev)
+        assert lib.axc_conv2d_minmax(table.handle, ctypes.byref(desc), xd.data_ptr(), fd.data_ptr(), *MM, y.data_ptr(),
+                                     ws.data_ptr(), ws.numel(), None) == 0
+        torch.cuda.synchronize()
+        jobs.append((desc, xd, fd, ws, out_shape, y.cpu().numpy()))
+    errors = []
+
+    def worker(which):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            mine = [jobs[2 * which], jobs[2 * which + 1]]
+            outs = [torch.empty(j[4], dtype=torch.float32, device=dev) for j in mine]
+            for it in range(150):
+                desc, xd, fd, ws, _, expect = mine[it & 1]
+                y = outs[it & 1]
+                rc = lib.axc_conv2d_minmax(table.handle, ctypes.byref(desc), xd.data_ptr(), fd.data_ptr(), *MM,
+                                           y.data_ptr(), ws.data_ptr(), ws.numel(), ctypes.c_void_p(stream.cuda_stream))
+                if rc != 0:
+                    errors.append((which, it, lib.axc_last_error()))
+                    return
+                if it % 25 == 24 or it >= 148:
+                    stream.synchronize()
+                    if not np.array_equal(y.cpu().numpy(), expect):
+                        errors.append((which, it, "result differs"))
+                        return
+            stream.synchronize()
+        except Exception as ex:  # noqa: BLE001 - reported through the list, the thread must not die silently
+            errors.append((which, -1, repr(ex)))
+
+    threads = [threading.Thread(target=worker, args=(w,)) for w in (0, 1)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
