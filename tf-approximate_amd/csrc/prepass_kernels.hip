@@ -902,7 +902,7 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 *filter_done = true;
             }
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(patch_sums_rows_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); // one value for every caller
             if (e != hipSuccess)
                 return e;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + g.N * bands)), dim3(block_threads),
