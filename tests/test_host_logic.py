@@ -202,3 +202,32 @@ def test_table_file_tool_round_trip_and_reference_format(pkg, golden_dir, tmp_pa
     assert stats["wrong_entries"] == 0 and stats["symmetric"]
     with pytest.raises(ValueError):
         tables.write_table(tmp_path / "bad.bin", np.zeros(10))
+
+
+def test_table_from_a_c_model(pkg, golden_dir, tmp_path):
+    """tables.py cmodel: a multiplier written in C is tabulated in the reference's order (input code outer).  An exact
+    model reproduces the reference's exact table byte for byte; an asymmetric model (drops the low bits of the
+    FILTER operand only) pins which argument is which."""
+    import subprocess
+    import sys
+    from tf_approximate_amd import tables
+    src = tmp_path / "models.c"
+    src.write_text("#include <stdint.h>\n"
+                   "uint64_t mul_exact(uint64_t a, uint64_t b) { return a * b; }\n"
+                   "uint16_t mul_drop(uint8_t a, uint8_t b) { return (uint16_t)(a * (b & 0xf0)); }\n")
+    exact = tables.table_from_c_model(str(src), "mul_exact")
+    assert exact.astype("<u2").tobytes() == open(os.path.join(golden_dir, "tables", "mul8u_1JFF.bin"), "rb").read()
+    drop = tables.table_from_c_model(str(src), "mul_drop", proto="u8").reshape(256, 256)
+    a = np.arange(256)[:, None]
+    b = np.arange(256)[None, :]
+    assert np.array_equal(drop, a * (b & 0xf0))
+    tool = os.path.join(os.path.dirname(golden_dir), "..", "tf-approximate_amd", "tables.py")
+    out = tmp_path / "drop.bin"
+    r = subprocess.run([sys.executable, tool, "cmodel", str(src), "mul_drop", str(out), "u8"], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    assert np.array_equal(tables.read_table(out).reshape(256, 256), drop)
+    with pytest.raises(RuntimeError, match="compiling"):
+        tables.table_from_c_model(str(src), "no_such_function")
+    with pytest.raises(ValueError):
+        tables.table_from_c_model(str(src), "mul exact")

@@ -7,8 +7,15 @@ entry [a * 256 + b] = approximate product of input code a and filter code b.
     python tables.py uniform SEED out.bin       # clamp(a*b + U(-64, 64))
     python tables.py tune in.bin out.bin        # the tf1 AxTune column remap (needs the built library)
     python tables.py info in.bin                # error statistics against exact multiplication
+    python tables.py cmodel model.c FUNC out.bin [u64|u8]
+                                                # compile a C model of a multiplier with gcc and tabulate FUNC(a, b);
+                                                # u64 (default): uint64_t FUNC(uint64_t, uint64_t), the EvoApproxLib
+                                                # form; u8: uint16_t FUNC(uint8_t, uint8_t)
 """
+import os
+import subprocess
 import sys
+import tempfile
 
 import numpy as np
 
@@ -34,6 +41,49 @@ def table_from_function(fn):
     a = np.arange(256, dtype=np.int64)[:, None]
     b = np.arange(256, dtype=np.int64)[None, :]
     return np.clip(np.broadcast_to(fn(a, b), (256, 256)), 0, 65535).astype(np.uint16).reshape(-1)
+
+
+_DRIVER = """#include <stdint.h>
+#include <stdio.h>
+%(proto)s;
+int main(int argc, char **argv)
+{
+    FILE *f = fopen(argv[1], "wb");
+    if (!f)
+        return 1;
+    for (unsigned a = 0; a < 256; a++)          /* input code outer, filter code inner: tf2/README.md:104-117 */
+        for (unsigned b = 0; b < 256; b++) {
+            uint16_t v = (uint16_t)%(func)s(a, b);
+            if (fwrite(&v, sizeof v, 1, f) != 1)
+                return 1;
+        }
+    return fclose(f) ? 1 : 0;
+}
+"""
+
+
+def table_from_c_model(source, func, proto="u64", cc="gcc"):
+    """Tabulates a C model of an 8x8 multiplier the way the reference's recipe does (tf2/README.md:104-117):
+    compiles `source` together with a generated driver and returns the 65536 products FUNC(a, b), a outer.
+    proto "u64": uint64_t FUNC(uint64_t, uint64_t) (the form of the EvoApproxLib models); "u8":
+    uint16_t FUNC(uint8_t, uint8_t)."""
+    if not func.isidentifier():
+        raise ValueError("not a C identifier: %r" % (func,))
+    protos = {"u64": "uint64_t %s(uint64_t, uint64_t)", "u8": "uint16_t %s(uint8_t, uint8_t)"}
+    if proto not in protos:
+        raise ValueError("proto must be u64 or u8")
+    with tempfile.TemporaryDirectory() as tmp:
+        driver = os.path.join(tmp, "driver.c")
+        with open(driver, "w") as f:
+            f.write(_DRIVER % {"proto": protos[proto] % func, "func": func})
+        exe = os.path.join(tmp, "tabulate")
+        r = subprocess.run([cc, "-O2", "-o", exe, driver, os.path.abspath(source)], stdout=subprocess.PIPE,
+                           stderr=subprocess.STDOUT, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("compiling %s failed:\n%s" % (source, r.stdout))
+        out = os.path.join(tmp, "table.bin")
+        subprocess.run([exe, out], check=True)
+        return read_table(out)
 
 
 def error_stats(table):
@@ -62,6 +112,11 @@ def main(argv):
     elif kind == "tune":
         from . import ops
         write_table(argv[3], ops.tune_table(read_table(argv[2])))
+    elif kind == "cmodel":
+        if len(argv) < 5:
+            print(__doc__)
+            return 2
+        write_table(argv[4], table_from_c_model(argv[2], argv[3], argv[5] if len(argv) > 5 else "u64"))
     elif kind == "info":
         for k, v in error_stats(read_table(argv[2])).items():
             print("%-16s %s" % (k, v))
