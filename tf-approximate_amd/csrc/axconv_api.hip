@@ -19,6 +19,24 @@ struct axc_table {
     int device;
 };
 
+namespace axc {
+int device_cus()
+{
+    static std::atomic<int> cached[64];   // per device; 0 = not asked yet
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return 256;
+    const int slot = dev & 63;
+    cus = cached[slot].load(std::memory_order_relaxed);
+    if (cus > 0)
+        return cus;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return 256;
+    cached[slot].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+} // namespace axc
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -273,14 +291,6 @@ ConvGeom make_geom(const axc_conv2d_dims &dm)
     return g;
 }
 
-int device_cus()
-{
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-        return 256;
-    return cus;
-}
 
 // Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
 // Derive cost per fill is constant; lookup cost per fill grows with the wavefront-rows a SIMD carries.

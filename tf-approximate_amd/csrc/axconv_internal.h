@@ -2,6 +2,9 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <map>
+#include <mutex>
+#include <utility>
 #include <stdint.h>
 #include <stddef.h>
 
@@ -119,6 +122,41 @@ __device__ inline uint32_t quantize_code(float v, float offset, float inv_scale)
     t = t < 255.0f ? t : 255.0f;      // truncation of [255,256) is 255 as well
     return (uint32_t)t;
 }
+
+// Function attributes belong to a (kernel, device) pair and never change here: they are set on first use instead
+// of before every launch (the runtime calls cost a few microseconds of host time each).
+inline hipError_t set_max_dynamic_lds_once(const void *kernel, int bytes, bool require_no_static_lds = false)
+{
+    static std::mutex mu;
+    static std::map<std::pair<const void *, int>, int> done;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return e;
+    const std::pair<const void *, int> key(kernel, dev);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = done.find(key);
+        if (it != done.end() && it->second >= bytes)
+            return hipSuccess;
+    }
+    if (require_no_static_lds) {
+        hipFuncAttributes attr;
+        e = hipFuncGetAttributes(&attr, kernel);
+        if (e != hipSuccess)
+            return e;
+        if (attr.sharedSizeBytes != 0)
+            return hipErrorInvalidConfiguration;
+    }
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess)
+        return e;
+    std::lock_guard<std::mutex> lock(mu);
+    done[key] = bytes;
+    return hipSuccess;
+}
+
+int device_cus();   // compute units of the current device (cached)
 
 // ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
 hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,

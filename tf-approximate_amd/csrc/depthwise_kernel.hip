@@ -225,8 +225,7 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
 template <typename Kernel, typename... Args>
 static hipError_t launch_with_table_lds(Kernel kernel, int grid, hipStream_t stream, Args... args)
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kTableBytes);
+    const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(kernel), kTableBytes);
     if (e != hipSuccess)
         return e;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBlockThreads), kTableBytes, stream, args...);
@@ -244,9 +243,7 @@ hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hi
         const int run = p.sw == 1 ? 32 : 16;
         const int nseg = (p.OW + run - 1) / run;
         const int seg_len = (p.OW + nseg - 1) / nseg;
-        int dev = 0, cus = 256;
-        if (hipGetDevice(&dev) == hipSuccess)
-            (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        const int cus = device_cus();
         const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;
         const int64_t blocks = (items + kBlockThreads - 1) / kBlockThreads;
         int g3 = (int)(blocks < cus ? blocks : cus);

@@ -519,15 +519,9 @@ static hipError_t launch_one(const DenseParams &p, hipStream_t stream)
 {
     auto kernel = lutgemm_expand_kernel<NT, OUT_I32>;
     // The generated assembly addresses LDS from offset 0: that holds as long as the kernel has no static LDS in
-    // front of its dynamic allocation.
-    hipFuncAttributes attr;
-    hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
-    if (e != hipSuccess)
-        return e;
-    if (attr.sharedSizeBytes != 0)
-        return hipErrorInvalidConfiguration;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDenseLdsBytes + kDenseParkBytes);
+    // front of its dynamic allocation (checked when the attribute is set, once per device).
+    const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(kernel),
+                                                  kDenseLdsBytes + kDenseParkBytes, true);
     if (e != hipSuccess)
         return e;
     hipLaunchKernelGGL(kernel, dim3(p.plan.grid), dim3(kDenseThreads), kDenseLdsBytes + kDenseParkBytes, stream, p);

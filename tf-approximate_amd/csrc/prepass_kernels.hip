@@ -901,8 +901,7 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                     lds = kFsLdsBytes;
                 *filter_done = true;
             }
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(patch_sums_rows_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); // one value for every caller
+            const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_rows_kernel), 160 * 1024);
             if (e != hipSuccess)
                 return e;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + g.N * bands)), dim3(block_threads),
@@ -938,8 +937,7 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
     const int sum_blocks = (fsum && filter) ? (int)blocks_for(g.Co, 64) : 0;
     const size_t lds = sum_blocks ? kFsLdsBytes : 0;
     if (lds) {
-        hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(filter_prep_kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kFsLdsBytes);
+        const hipError_t ea = set_max_dynamic_lds_once(reinterpret_cast<const void *>(filter_prep_kernel), kFsLdsBytes);
         if (ea != hipSuccess)
             return ea;
     }
