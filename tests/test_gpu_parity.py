@@ -481,3 +481,29 @@ def test_concurrent_host_threads_through_the_c_abi(pkg, oracle):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def test_python_wrapper_on_two_streams(pkg, oracle):
+    """Calls issued alternately on two torch streams may overlap on the GPU: the wrapper keeps a workspace per
+    stream, so both must still give the results of a lone call."""
+    dev = gpu_util.dev()
+    table = pkg.synth.table_random(29)
+    ops_, ins, expect = [], [], []
+    for i, (xs, fs) in enumerate([((4, 40, 40, 32), (3, 3, 32, 64)), ((4, 36, 36, 48), (3, 3, 48, 32))]):
+        x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=60 + i)
+        op = pkg.ApproxConv2DWithMinMaxVars([1, 1, 1, 1], 8, table, "SAME")
+        xd, fd = torch.from_numpy(x).to(dev), torch.from_numpy(f).to(dev)
+        ops_.append(op)
+        ins.append((xd, fd))
+        expect.append(op(xd, fd, *MM).cpu().numpy())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)]
+    outs = [None, None]
+    for it in range(40):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                outs[i] = ops_[i](*ins[i], *MM)
+    for s in streams:
+        s.synchronize()
+    for i in (0, 1):
+        assert np.array_equal(outs[i].cpu().numpy(), expect[i])

@@ -153,6 +153,8 @@ NETWORKS = {
     # name: (program builder, input shape, input range)
     "cifar_resnet_b128": (cifar_resnet_program, (128, 32, 32, 3), (0.0, 1.0)),
     "resnet50_b64": (resnet50_program, (64, 224, 224, 3), (0.0, 1.0)),
+    "resnet50_b8": (resnet50_program, (8, 224, 224, 3), (0.0, 1.0)),
+    "resnet50_b1": (resnet50_program, (1, 224, 224, 3), (0.0, 1.0)),
     "inverted_residual_b64_s1": (lambda: inverted_residual_program(32, 6, 1), (64, 112, 112, 32), (-1.0, 1.0)),
     "inverted_residual_b64_s2": (lambda: inverted_residual_program(32, 6, 2), (64, 112, 112, 32), (-1.0, 1.0)),
 }

@@ -113,10 +113,13 @@ _workspaces = {}
 
 
 def _workspace(device, nbytes):
-    buf = _workspaces.get(device)
+    """Scratch memory of a call, cached per (device, current stream): calls issued on one stream run in order and
+    may share it; calls on different streams may overlap and must not."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
-        _workspaces[device] = buf
+        _workspaces[key] = buf
     return buf
 
 
