@@ -22,9 +22,10 @@ barriers.  The macro interleaves, in one instruction stream with hand-counted s_
   derive    the staged rows of fill p+1 (buffer BUF^1) are transposed into expanded-row buffer BUF^1: two
             items per lane, each four 8-byte reads, eight v_perm_b32 and four 8-byte writes.
             Stage, loads and derive are cut into micro-operations and one of them is slotted in behind every
-            16-byte chunk of the lookups, so that the memory pipeline and the LDS see them spread out instead
-            of as one burst per wavefront right after the barrier; what a wavefront with few pixels has not
-            placed by its last chunk follows behind it.
+            16-byte chunk of the lookups (loads first, so that their latency runs under the lookups), so that
+            the memory pipeline and the LDS see them spread out instead of as one burst per wavefront right
+            after the barrier; what a wavefront with few pixels has not placed by its last chunk follows
+            behind it.
 
 NT = 16: a fill holds 4 input channels and the activation dword is used as it is.
 NT = 32 / 64: a fill holds 2 / 1 channels; the dword is first rotated right by SHIFT bits (an SGPR) so that
@@ -185,14 +186,19 @@ def emit(nt, buf):
     def both(f, g):
         return lambda st, state: (f(st, state), g(st, state))
 
-    # reads of a derive item are issued nine slots before its transposes
-    aux = [derive_reads(0)]
+    # Global loads first: a wavefront with few pixels has few chunk slots, and what does not fit behind a chunk is
+    # issued behind the last one, right in front of the wait for it.  Then the expansion of fill p+1, the reads of
+    # a derive item five slots ahead of its transposes.
+    aux = []
     for j in range(4):
-        aux += [stage_write(j), row_load(j)]
-    aux += [both(derive_consume(0), derive_reads(1))]
-    aux += [code_load(j) for j in range(4)]
+        aux += [both(stage_write(j), row_load(j))]      # row_load j reuses the registers stage_write j empties,
+    aux += [both(code_load(0), code_load(1)), both(code_load(2), code_load(3))]   # code_load j those of row_load j
     aux += [both(act_load(r), act_load(r + 1)) for r in range(0, rows, 2)]
-    while len(aux) < 18:
+    aux += [derive_reads(0)]
+    for _ in range(4):
+        aux.append(lambda st, state: None)
+    aux += [both(derive_consume(0), derive_reads(1))]
+    for _ in range(4):
         aux.append(lambda st, state: None)
     aux += [derive_consume(1)]
 
