@@ -1,0 +1,143 @@
+"""The generated phase body (tf-approximate_amd/csrc/gen_lookup_asm.py) waits for LDS and memory operations with
+hand-counted s_waitcnt.  This test re-reads the emitted instruction text with an independent model of the hardware
+counters (LDS operations and vector-memory loads each complete in issue order; s_waitcnt N lets the newest N stay
+in flight; lgkmcnt is a 4-bit counter) and checks, on every control-flow path of every macro, that no instruction
+touches a register an outstanding load has yet to write, that the counter never needs more than 15, and that
+nothing is in flight when the macro ends."""
+import importlib.util
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOKEN = re.compile(r"%\[\w+\]|v\[\d+:\d+\]|v\d+")
+
+
+def _generator():
+    path = os.path.join(ROOT, "tf-approximate_amd", "csrc", "gen_lookup_asm.py")
+    spec = importlib.util.spec_from_file_location("gen_lookup_asm", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def _instructions(macro_text):
+    """The quoted assembly lines of the macro, in order: ("label", name) or ("ins", text)."""
+    out = []
+    for m in re.finditer(r'"([^"]*)\\n\\t"', macro_text):
+        text = m.group(1).strip()
+        if text.endswith(":"):
+            out.append(("label", text[:-1]))
+        else:
+            out.append(("ins", text))
+    return out
+
+
+def _regs(token):
+    if token.startswith("v["):
+        a, b = token[2:-1].split(":")
+        return ["v%d" % i for i in range(int(a), int(b) + 1)]
+    return [token]
+
+
+def _operands(text):
+    regs = []
+    for tok in TOKEN.findall(text):
+        regs += _regs(tok)
+    return regs
+
+
+def _paths(prog):
+    """Every way through the macro: conditional branches are followed both ways."""
+    labels = {name: i for i, (kind, name) in enumerate(prog) if kind == "label"}
+    done, stack = [], [(0, [])]
+    while stack:
+        pc, trace = stack.pop()
+        trace = list(trace)
+        while pc < len(prog):
+            kind, text = prog[pc]
+            if kind == "ins":
+                op = text.split()[0]
+                if op == "s_branch":
+                    pc = labels[text.split()[1]]
+                    continue
+                if op.startswith("s_cbranch"):
+                    stack.append((labels[text.split()[1]], list(trace)))
+                else:
+                    trace.append(text)
+            pc += 1
+        done.append(trace)
+    return done
+
+
+def _check_path(trace):
+    lds, vm = [], []          # in-flight operations, oldest first: the set of registers each will write
+    for text in trace:
+        op = text.split()[0]
+        if op == "s_waitcnt":
+            for name, queue in (("lgkmcnt", lds), ("vmcnt", vm)):
+                m = re.search(name + r"\((\d+)\)", text)
+                if m:
+                    del queue[:max(0, len(queue) - int(m.group(1)))]
+            continue
+        touched = _operands(text)
+        pending = set().union(*lds, *vm) if (lds or vm) else set()
+        clash = pending.intersection(touched)
+        assert not clash, "%r touches %s while a load into it is in flight" % (text, sorted(clash))
+        if op.startswith("ds_"):
+            first = TOKEN.search(text).group(0)
+            lds.append(set(_regs(first)) if op.startswith("ds_read") else set())
+            assert len(lds) <= 15, "more than 15 LDS operations in flight at %r" % text
+        elif op.startswith("buffer_load"):
+            vm.append(set(_regs(TOKEN.search(text).group(0))))
+    assert not lds and not vm, "operations still in flight at the end of the macro"
+
+
+@pytest.mark.parametrize("nt", [16, 32, 64])
+@pytest.mark.parametrize("buf", [0, 1])
+def test_every_path_waits_for_what_it_uses(nt, buf):
+    gen = _generator()
+    prog = _instructions(gen.emit(nt, buf))
+    assert sum(1 for kind, text in prog if kind == "ins" and text.startswith("ds_read_b128")) >= 8
+    paths = _paths(prog)
+    rows = 2 * (64 // nt)
+    assert len(paths) == rows + 1        # 0 pixels, or the last pixel is pixel 0 .. rows-1
+    for trace in paths:
+        _check_path(trace)
+    # a lane with r pixels issues 8 lookups per pixel
+    counts = sorted(sum(1 for t in trace if t.startswith("ds_read_b128")) for trace in paths)
+    assert counts == [8 * r for r in range(rows + 1)]
+
+
+def test_the_model_notices_a_missing_wait():
+    """The checker itself: dropping one s_waitcnt from a path must be reported."""
+    gen = _generator()
+    prog = _instructions(gen.emit(16, 0))
+    path = max(_paths(prog), key=len)
+    first_wait = next(i for i, t in enumerate(path) if t.startswith("s_waitcnt lgkmcnt"))
+    broken = path[:first_wait] + path[first_wait + 1:]
+    with pytest.raises(AssertionError):
+        _check_path(broken)
+
+
+@pytest.mark.parametrize("nt", [16, 32, 64])
+def test_every_accumulator_gets_its_share_of_a_fill(nt):
+    """A fill holds 64 / NT input channels for each of NT columns: on the path of a full lane every accumulator of
+    every pixel must receive exactly that many table entries, half of the columns from the low halves of the dwords
+    (plain add of the dword) and half from the high halves (SDWA WORD_1)."""
+    gen = _generator()
+    rows = 2 * (64 // nt)
+    path = max(_paths(_instructions(gen.emit(nt, 0))), key=len)
+    adds = {}
+    for text in path:
+        if text.startswith("v_add_u32"):
+            dst = TOKEN.search(text).group(0)
+            if dst.startswith("%[c"):
+                adds.setdefault(dst, []).append("WORD_1" in text)
+    assert len(adds) == rows * nt
+    for r in range(rows):
+        for j in range(nt):
+            kinds = adds["%%[c%d_%d]" % (r, j)]
+            assert len(kinds) == 64 // nt
+            assert all(k == bool(j & 1) for k in kinds)
