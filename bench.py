@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 
 NOMINAL_LDS_LOOKUPS_PER_S = 256 * 32 * 2.4e9
 HBM_PEAK_GBPS = 8000.0
+PREROLL_S = 0.3
 
 WORKLOADS = {
     # name: (x_shape, f_shape, strides, depthwise)
@@ -126,6 +127,13 @@ def main():
     fd = torch.from_numpy(f).to(dev)
     op = pkg.ApproxConv2DWithMinMaxVars([1, strides[0], strides[1], 1], 8, table, "SAME", depthwise=depthwise)
 
+    # Settle the clocks first, whatever W is: the GPU needs a few hundred milliseconds of load before it runs at its
+    # sustained frequency (the first calls are ~10 % slower).  Not counted as warm-up steps; reported as preroll_s.
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < PREROLL_S:
+        for _ in range(20):
+            y = op(xd, fd, *mm)
+        torch.cuda.synchronize()
     for _ in range(max(args.warmup, 1)):
         y = op(xd, fd, *mm)
     torch.cuda.synchronize()
@@ -247,6 +255,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preroll_s": PREROLL_S,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
