@@ -63,3 +63,28 @@ def test_random_layer_entry_point_vs_composition(pkg, oracle, seed):
     if seed % 2:
         y_ref = np.maximum(y_ref, 0.0)
     assert refimpl.linf_rel(y, y_ref) <= 1e-5, (xs, fs, strides, dil, padding)
+
+
+EXTREMES = [
+    ((2, 7, 7, 512), (1, 1, 512, 4096), (1, 1), (1, 1), "SAME"),    # 256 column tiles
+    ((1, 5, 5, 3600), (3, 3, 3600, 8), (1, 1), (1, 1), "VALID"),    # K = 32400, just below the int32 bound
+    ((1, 300, 3, 4), (3, 3, 4, 16), (1, 1), (1, 1), "SAME"),        # tall and narrow
+    ((1, 3, 1000, 4), (1, 7, 4, 16), (1, 2), (1, 1), "SAME"),       # flat and wide, strided along the row
+    ((3, 64, 64, 1), (5, 5, 1, 1), (1, 1), (2, 2), "SAME"),         # one channel in, one column out, dilated
+    ((1, 1, 1, 1), (1, 1, 1, 1), (1, 1), (1, 1), "VALID"),          # a single product
+    ((70, 9, 9, 8), (3, 3, 8, 24), (2, 2), (1, 1), "VALID"),        # many small images
+]
+
+
+@pytest.mark.parametrize("case", EXTREMES, ids=[str(i) for i in range(len(EXTREMES))])
+def test_extreme_shapes_vs_oracle(pkg, oracle, case):
+    xs, fs, strides, dil, padding = case
+    mm = (-1.0, 1.0, -0.5, 0.5)
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, mm, seed=7)
+    table = pkg.synth.table_random(9)
+    y, acc = gpu_util.run_op(pkg, table, x, f, mm, strides, padding, dil)
+    rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding, dilations=dil,
+                                            threads=8)
+    assert rc == 0
+    assert np.array_equal(acc, acc_ref), case
+    assert refimpl.linf_rel(y, y_ref) <= 1e-5, case
