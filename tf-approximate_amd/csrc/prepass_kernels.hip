@@ -452,6 +452,97 @@ __global__ void __launch_bounds__(kFsThreads) filter_prep_kernel(const float *__
     filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, q, wq);
 }
 
+// Patch sums of a 1x1, stride-1, unpadded layer: the patch of an output pixel is the pixel itself, so the pixels
+// of the whole batch form one flat list and no window or halo exists.  A workgroup takes up to kFlatPixels consecutive
+// pixels and walks their channels in chunks of kFlatChunk: all threads copy a chunk into LDS (and quantize it
+// into the code layout on the way, when xq is given), then one thread per pixel extends its sequential sum by the
+// chunk's channels.  With many channels this keeps 256 sums going per workgroup where a band of image rows in
+// LDS would hold one row's worth.  The loads of the next chunk are in flight while the current one is summed.
+constexpr int kFlatPixels = 256, kFlatChunk = 64, kFlatThreads = 512;
+constexpr int kFlatPitch = kFlatChunk + 4;                         // floats per pixel in LDS
+constexpr int kFlatPer = kFlatPixels * (kFlatChunk / 4) / kFlatThreads; // 16-byte loads per thread and chunk
+
+__device__ __forceinline__ void patch_sums_flat_body(const float *__restrict__ x, const ConvGeom &g,
+                                                     const TensorQuant &tq, const LayerQuant *__restrict__ lq_dev,
+                                                     float *__restrict__ psum, uint32_t *__restrict__ xq,
+                                                     const int bid, const int pixels)
+{
+    // pixels: pixels per workgroup, 64 / 128 / 256 (fewer when the layer has few pixels, for enough workgroups)
+    const TensorQuant qt = lq_dev ? lq_dev->in : tq;
+    if (xq && bid == 0)
+        for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
+            xq[(int64_t)g.N * g.H * g.C4 * g.W + i] = qt.zp4;
+    extern __shared__ __align__(16) unsigned char pf_lds[];
+    float *const rows = reinterpret_cast<float *>(pf_lds);
+    const int t = threadIdx.x;
+    const int64_t m0 = (int64_t)bid * pixels;
+    const int npx = (int)(g.M - m0 < pixels ? g.M - m0 : pixels);
+    // thread -> (channel quad of the chunk, pixel) once: quad q of pixels px0, px0 + 32, ...
+    constexpr int QUADS = kFlatChunk / 4, PSTEP = kFlatThreads / QUADS;
+    const int q = t % QUADS, px0 = t / QUADS;
+    const bool copier = t < kFlatThreads;
+    uint32_t xq_idx[kFlatPer];        // dword index in xq of (pixel, quad q of chunk 0)
+    int64_t x_idx[kFlatPer];          // float index in x of the same
+#pragma unroll
+    for (int k = 0; k < kFlatPer; ++k) {
+        const int px = px0 + k * PSTEP;    // k beyond pixels / PSTEP: px >= npx, nothing loaded or stored
+        const int64_t m = m0 + (px < npx ? px : 0);
+        const int64_t nh = m / g.W;
+        const int w = (int)(m - nh * g.W);
+        xq_idx[k] = (uint32_t)((nh * g.C4 + q) * g.W + w);
+        x_idx[k] = m * g.C + q * 4;
+    }
+    const int chunks = (g.C + kFlatChunk - 1) / kFlatChunk;
+    float4 v[kFlatPer];
+    auto load_chunk = [&](int c0) {
+#pragma unroll
+        for (int k = 0; k < kFlatPer; ++k) {
+            v[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (copier && px0 + k * PSTEP < npx && c0 + q * 4 < g.C)
+                v[k] = *reinterpret_cast<const float4 *>(x + x_idx[k] + c0);
+        }
+    };
+    load_chunk(0);
+    float s = 0.0f;
+    for (int ch = 0; ch < chunks; ++ch) {
+        const int c0 = ch * kFlatChunk;
+        if (copier) {
+#pragma unroll
+            for (int k = 0; k < kFlatPer; ++k) {
+                const int px = px0 + k * PSTEP;
+                if (px >= pixels)
+                    continue;
+                const float4 f = fake_quant_value4(v[k], qt);
+                *reinterpret_cast<float4 *>(&rows[px * kFlatPitch + q * 4]) = f;
+                if (xq && px < npx && c0 + q * 4 < g.C)
+                    xq[xq_idx[k] + (uint32_t)(c0 / 4) * (uint32_t)g.W] =
+                        phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
+                        (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
+                        (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
+                        (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
+            }
+        }
+        __syncthreads();
+        if (ch + 1 < chunks)
+            load_chunk(c0 + kFlatChunk);
+        if (t < npx) {
+            const int nq = (g.C - c0 < kFlatChunk ? g.C - c0 : kFlatChunk) / 4;
+            const float *src = &rows[t * kFlatPitch];
+#pragma unroll 8
+            for (int qq = 0; qq < nq; ++qq) {
+                const float4 f = *reinterpret_cast<const float4 *>(src + qq * 4);
+                s = __fadd_rn(s, f.x);
+                s = __fadd_rn(s, f.y);
+                s = __fadd_rn(s, f.z);
+                s = __fadd_rn(s, f.w);
+            }
+        }
+        __syncthreads();
+    }
+    if (t < npx)
+        psum[m0 + t] = s;
+}
+
 // The filter pre-pass of a layer is independent of its input pre-pass: as two launches they would run one after
 // the other, so the launch below carries both.  The first filter_blocks8 workgroups (a multiple of 8, which keeps
 // workgroup index mod 8 = XCD for the others) do the filter work of filter_prep_kernel, the rest the patch sums.
@@ -486,6 +577,10 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
         }
         const int64_t i = (int64_t)((int)blockIdx.x - fw.sum_blocks) * blockDim.x + threadIdx.x;
         filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+        return;
+    }
+    if (rb == 0) { // 1x1, stride 1: flat pixel list
+        patch_sums_flat_body(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8, in_rows);
         return;
     }
     patch_sums_rows_body(x, g, rb, in_rows, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
@@ -863,18 +958,27 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
             rb = cand;
             in_rows = rows_needed;
         }
-        if (rb > 0) {
+        // 1x1, stride 1, no padding, and a band would hold few pixels (many channels): the flat-list variant
+        const bool flat = g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 &&
+                          rb * g.OW < 192;
+        if (flat) { // in_rows carries the pixels per workgroup: at least ~2 workgroups per CU where the layer allows
+            rb = 0;
+            in_rows = g.M >= 512 * kFlatPixels ? kFlatPixels : (g.M >= 512 * 128 ? 128 : 64);
+        }
+        if (rb > 0 || flat) {
             int threads = ((rb * g.OW + 63) / 64) * 64;
             threads = threads < 512 ? 512 : threads;   // the copy into LDS wants more threads than there are pixels
             // Band b owns input rows [b*rb*sh, (b+1)*rb*sh), the last band up to H.  They are quantized by the
             // block that holds them if every band's window (rows b*rb*sh - ph onwards, in_rows of them) contains
             // its owned rows, the last window reaches the last image row, and the fast copy loop is in use.
-            const bool fuse = xq_fused && fused && g.sh - 1 + g.ph <= (g.KH - 1) * g.dh &&
-                              (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0;
+            const bool fuse = xq_fused && fused &&
+                              (flat || (g.sh - 1 + g.ph <= (g.KH - 1) * g.dh &&
+                                        (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0));
             if (fuse)
                 *fused = true;
-            size_t lds = (size_t)in_rows * row_bytes;
-            const int bands = (g.OH + rb - 1) / rb;
+            size_t lds = flat ? (size_t)in_rows * kFlatPitch * 4 : (size_t)in_rows * row_bytes;
+            const int bands = flat ? 0 : (g.OH + rb - 1) / rb;
+            const int64_t work_blocks = flat ? (g.M + in_rows - 1) / in_rows : (int64_t)g.N * bands;
             // the filter pre-pass rides along in the same launch (its workgroups want 512 or 1024 threads, so
             // every workgroup gets that many; only `threads` of them take part in the patch sums)
             FilterWork fw = {};
@@ -904,7 +1008,7 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
             const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_rows_kernel), 160 * 1024);
             if (e != hipSuccess)
                 return e;
-            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + g.N * bands)), dim3(block_threads),
+            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)), dim3(block_threads),
                                lds, stream, x, g, rb, in_rows, threads, tq, lq_dev, psum, fuse ? xq_fused : nullptr, fw);
             return hipGetLastError();
         }
