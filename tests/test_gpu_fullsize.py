@@ -101,7 +101,7 @@ def test_north_star_layer_is_deterministic(pkg, north_star):
     assert np.array_equal(acc0, acc1) and np.array_equal(y0, y1)
 
 
-@pytest.mark.parametrize("name", ["A_1x1_256_1024", "B_3x3_512_512", "stem_7x7", "stage4_3x3"])
+@pytest.mark.parametrize("name", ["A_1x1_256_1024", "B_3x3_512_512", "stem_7x7", "stage4_3x3", "reduce_1x1_256_64"])
 @pytest.mark.parametrize("tname", ["random", "exact"])
 def test_stress_layers_sampled_pixels(pkg, oracle, name, tname):
     """The large GEMM-dominated stress layers (A: 1x1 32x56x56x256->1024; B: 3x3 64x28x28x512->512, K = 4608) and the
@@ -111,6 +111,7 @@ def test_stress_layers_sampled_pixels(pkg, oracle, name, tname):
         "B_3x3_512_512": ((64, 28, 28, 512), (3, 3, 512, 512), (1, 1)),
         "stem_7x7": ((16, 224, 224, 3), (7, 7, 3, 64), (2, 2)),
         "stage4_3x3": ((64, 7, 7, 512), (3, 3, 512, 512), (1, 1)),
+        "reduce_1x1_256_64": ((64, 56, 56, 256), (1, 1, 256, 64), (1, 1)),   # flat pre-pass, 256 pixels per workgroup
     }
     xs, fs, strides = shapes[name]
     x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=len(name), codes="halfnormal")
