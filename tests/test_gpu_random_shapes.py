@@ -88,3 +88,30 @@ def test_extreme_shapes_vs_oracle(pkg, oracle, case):
     assert rc == 0
     assert np.array_equal(acc, acc_ref), case
     assert refimpl.linf_rel(y, y_ref) <= 1e-5, case
+
+
+@pytest.mark.parametrize("columns", [32, 64])
+def test_wider_column_tiles_vs_oracle(pkg, oracle, columns, monkeypatch):
+    """The tile planner has so far always chosen 16-column tiles; the 32- and 64-column variants of the kernel
+    (other accumulator shapes, rotated activation dwords, the untransposed store path for 64) are pinned here by
+    forcing the width through the environment."""
+    monkeypatch.setenv("AXC_TILE_COLUMNS", str(columns))
+    mm = (-1.0, 1.0, -0.5, 0.5)
+    cases = [((2, 24, 24, 16), (3, 3, 16, 64), (1, 1), (1, 1), "SAME"),
+             ((1, 17, 19, 8), (1, 1, 8, 48), (2, 2), (1, 1), "SAME"),
+             ((2, 15, 15, 12), (5, 5, 12, 100), (1, 1), (1, 1), "VALID"),
+             ((4, 40, 40, 64), (3, 3, 64, 64), (1, 1), (1, 1), "SAME"),
+             ((1, 30, 30, 4), (3, 3, 4, 70), (2, 2), (1, 1), "SAME"),
+             ((3, 9, 9, 5), (3, 3, 5, 33), (1, 1), (2, 2), "SAME"),
+             ((8, 56, 56, 64), (1, 1, 64, 256), (1, 1), (1, 1), "SAME")]
+    for xs, fs, strides, dil, padding in cases:
+        plan = pkg.ops.conv2d_tile_plan(xs, fs, [1, strides[0], strides[1], 1], padding)
+        assert plan["columns_per_tile"] == columns
+        x, f, _, _ = refimpl.grid_case(pkg, xs, fs, mm, seed=3)
+        table = pkg.synth.table_random(9)
+        y, acc = gpu_util.run_op(pkg, table, x, f, mm, strides, padding, dil)
+        rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding, dilations=dil,
+                                                threads=8)
+        assert rc == 0
+        assert np.array_equal(acc, acc_ref), (columns, xs, fs)
+        assert refimpl.linf_rel(y, y_ref) <= 1e-5, (columns, xs, fs)

@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <string>
@@ -299,9 +300,18 @@ DensePlan make_plan(const ConvGeom &g, int cus)
     DensePlan best{};
     double best_cost = 1e300;
     const int taps = g.KH * g.KW;
+    // AXC_TILE_COLUMNS=16|32|64 pins the tile width (for tests of the wider tiles and for experiments; the cost
+    // model itself has so far always preferred 16 on this GPU)
+    int forced_nt = 0;
+    if (const char *env = std::getenv("AXC_TILE_COLUMNS"))
+        forced_nt = std::atoi(env);
     for (int nt : {16, 32, 64}) {
-        if (nt > 16 && nt / 2 >= g.Co)
+        if (forced_nt == 16 || forced_nt == 32 || forced_nt == 64) {
+            if (nt != forced_nt)
+                continue;
+        } else if (nt > 16 && nt / 2 >= g.Co) {
             continue; // half the columns of a wider tile would be padding
+        }
         const int R = 2 * (64 / nt), ks = 64 / nt, subs = 4 / ks;
         const int n_col = (g.Co + nt - 1) / nt;
         const int fills = taps * g.C4 * subs;
