@@ -149,22 +149,24 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     const rsrc_t tab_rsrc = make_rsrc(p.tableT, (uint32_t)kTableAllocBytes);
     (void)taps;
 
-    for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        // Workgroups are handed to the 8 XCDs round-robin, and each XCD has its own L2.  The column tiles of one
-        // row tile read the same activations, so they go to the same XCD, next to each other in time:
-        // inside a group of 8 * n_col_tiles consecutive tiles, tile r is (row tile r % 8, column tile r / 8).
-        int ct, rt;
-        {
-            const int nct = nct_v, group = 8 * nct;
-            const int gi = tile / group, r = tile - gi * group;
-            if ((gi + 1) * group <= ntiles) {
-                ct = r >> 3;
-                rt = gi * 8 + (r & 7);
-            } else { // the ragged tail keeps the plain order
-                ct = tile % nct;
-                rt = tile / nct;
-            }
-        }
+    // Tiles in the order (row tile, column tile incl. K split), column tile fastest; a workgroup takes a contiguous
+    // run of them, so that its consecutive tiles mostly share their row tile: same pixels, same parked geometry,
+    // same activations.  Workgroups are handed to the 8 XCDs round-robin, and each XCD has its own L2: the runs
+    // are dealt so that neighbouring runs, which share row tiles too, go to workgroups of one XCD.
+    int run_first, run_count;
+    {
+        const int G = (int)gridDim.x;
+        const int w = (G & 7) == 0 ? ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
+        const int per = ntiles / G, extra = ntiles - per * G;
+        run_first = w * per + (w < extra ? w : extra);
+        run_count = per + (w < extra ? 1 : 0);
+    }
+    int prev_rt = -1;
+    bool rvalid[DenseCfg<NT>::R];    // this lane's pixel exists
+    uint32_t nr = 0;                 // pixels of this lane whose wavefront row exists (a prefix; wave-uniform)
+    for (int tile = run_first; tile < run_first + run_count; ++tile) {
+        const int rt = tile / nct_v;
+        int ct = tile - rt * nct_v;
         const int ksi = ct / p.plan.n_col_tiles;           // K split of this tile
         ct -= ksi * p.plan.n_col_tiles;
         const int f0 = ksi * p.plan.fills_per_split;        // its fills: [f0, f0 + fills)
@@ -183,32 +185,35 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         const int wr_base = old_half ? wave : wr_old + wave - kDenseWaves / 2; // then every fourth wavefront-row
         const int64_t wr_end = row0 + (int64_t)(old_half ? wr_old : wrows) * 64;
 
-        // ---- per-pixel geometry (parked in LDS; only read back when the tap changes) ----
-        bool rvalid[R];    // this lane's pixel exists
-        uint32_t nr = 0;   // pixels of this lane whose wavefront row exists (a prefix; wave-uniform)
+        // ---- per-pixel geometry (parked in LDS, in slots private to the thread; only read back when the tap
+        // changes).  It depends on the row tile alone: kept from the previous tile when that had the same one.
+        if (rt != prev_rt) {
+            prev_rt = rt;
+            nr = 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int64_t wrow = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
-            nr += (wrow < row_end && wrow < wr_end) ? 1u : 0u;
-            const int64_t m = wrow + lane;
-            rvalid[r] = m < row_end && wrow < wr_end;
-            const int64_t mm = rvalid[r] ? m : row0;
-            int n, rem;
-            if (g.M <= 0x7fffffff) { // the usual case: 32-bit divisions (a 64-bit one costs several times more)
-                const uint32_t ohow = (uint32_t)(g.OH * g.OW);
-                n = (int)((uint32_t)mm / ohow);
-                rem = (int)((uint32_t)mm - (uint32_t)n * ohow);
-            } else {
-                n = (int)(mm / ((int64_t)g.OH * g.OW));
-                rem = (int)(mm - (int64_t)n * g.OH * g.OW);
+            for (int r = 0; r < R; ++r) {
+                const int64_t wrow = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
+                nr += (wrow < row_end && wrow < wr_end) ? 1u : 0u;
+                const int64_t m = wrow + lane;
+                rvalid[r] = m < row_end && wrow < wr_end;
+                const int64_t mm = rvalid[r] ? m : row0;
+                int n, rem;
+                if (g.M <= 0x7fffffff) { // the usual case: 32-bit divisions (a 64-bit one costs several times more)
+                    const uint32_t ohow = (uint32_t)(g.OH * g.OW);
+                    n = (int)((uint32_t)mm / ohow);
+                    rem = (int)((uint32_t)mm - (uint32_t)n * ohow);
+                } else {
+                    n = (int)(mm / ((int64_t)g.OH * g.OW));
+                    rem = (int)(mm - (int64_t)n * g.OH * g.OW);
+                }
+                const int oh = (int)((uint32_t)rem / (uint32_t)g.OW);
+                const int ow = rem - oh * g.OW;
+                const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
+                // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
+                park[(2 * r) * kDenseThreads] = (uint32_t)((n * g.H + ih0) * rowstep + iw0);
+                // input coordinates of tap (0, 0); ih0 = -32768 marks a pixel that does not exist
+                park[(2 * r + 1) * kDenseThreads] = rvalid[r] ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
             }
-            const int oh = (int)((uint32_t)rem / (uint32_t)g.OW);
-            const int ow = rem - oh * g.OW;
-            const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
-            // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
-            park[(2 * r) * kDenseThreads] = (uint32_t)((n * g.H + ih0) * rowstep + iw0);
-            // input coordinates of tap (0, 0); ih0 = -32768 marks a pixel that does not exist
-            park[(2 * r + 1) * kDenseThreads] = rvalid[r] ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
         }
 
         const uint32_t wq_tile = ((uint32_t)ct * (uint32_t)fills_all + (uint32_t)f0) * 128u; // this tile's first codes
