@@ -42,7 +42,7 @@ DEFAULT = "conv3x3_b64_56x56x64_to_64_s1_same"
 # HBM bytes per launch of the main kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
 # scaled by what the same counter reads for --copy-calibration (profiles/lutgemm_expand_conv3x3_b64_56x56x64.md).
 MEASURED_TRAFFIC_BYTES = {
-    "conv3x3_b64_56x56x64_to_64_s1_same": 2.000 * 13743.5 * 1024 + 1.000 * 70194.6 * 1024,
+    "conv3x3_b64_56x56x64_to_64_s1_same": 2.000 * 13465.0 * 1024 + 1.000 * 72175.1 * 1024,
     # profiles/depthwise_lut3x3_dw3x3_b64_112x112x192_s1.md
     "dw3x3_b64_112x112x192_s1": 2.000 * 838534 * 1024 + 1.000 * 602112 * 1024,
 }
