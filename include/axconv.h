@@ -136,6 +136,20 @@ int axc_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc,
                       float input_min, float input_max, float filter_min, float filter_max,
                       float *output, void *workspace, size_t workspace_bytes, void *stream);
 
+/* axc_conv2d_minmax for callers that cannot allocate or own a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose launcher allocates its
+ * temporaries per call (approx_nn_conv_ops.cpp:590-613).  The workspace is a fixed array of
+ * axc_conv2d_static_workspace_limit() bytes (32 MiB) inside the library's device image, one copy per GPU, held
+ * until the process ends; the call itself allocates and frees nothing.  Layers whose
+ * axc_conv2d_workspace_bytes exceeds the limit are refused with AXC_INVALID_ARGUMENT.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (two streams, two threads) race; issue them on one stream.
+ * Results are identical to axc_conv2d_minmax. */
+int axc_conv2d_static_workspace_limit(size_t *bytes);
+int axc_conv2d_minmax_static(const axc_table *table, const axc_conv2d_desc *desc,
+                             const float *input, const float *filter,
+                             float input_min, float input_max, float filter_min, float filter_max,
+                             float *output, void *stream);
+
 /* Depthwise variant (filter [rows, cols, C, 1]).  The reference has none: its CPU launcher rejects
  * in_depth != filter in_depth (approx_nn_conv_ops.cpp:229-232).  Defined as the dense op applied to
  * every channel on its own with the tensor-wide min/max. */

@@ -58,6 +58,8 @@ SYMBOLS = [
     ("axc_depthwise_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
+    ("axc_conv2d_static_workspace_limit", ctypes.c_int, [ctypes.POINTER(_sz)]),
+    ("axc_conv2d_minmax_static", ctypes.c_int, [_vp, _desc, _vp, _vp, _f, _f, _f, _f, _vp, _vp]),
     ("axc_fake_approx_conv2d", ctypes.c_int, [_vp, _desc, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
     ("axc_axconv2d_quint8", ctypes.c_int, [_vp, _desc, _vp, _vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp, _sz, _vp]),
     ("axc_table_tune_weights", ctypes.c_int, [_vp, _vp]),

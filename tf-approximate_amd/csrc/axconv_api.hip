@@ -20,6 +20,12 @@ struct axc_table {
     int device;
 };
 
+// Workspace of axc_conv2d_minmax_static: a fixed array in the library's device image, one copy per GPU, held until
+// the process ends.  In host code this name is only a handle for hipGetSymbolAddress; the address each device
+// reports is what kernels and copies get.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace axc {
 int device_cus()
 {
@@ -60,6 +66,29 @@ int fail_hip(hipError_t e, const char *what)
         if (e_ != hipSuccess)                        \
             return fail_hip(e_, #call);              \
     } while (0)
+
+// Device address of `scratch` on the current device, looked up once per device with that device current.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **ptr)
+{
+    int dev = 0;
+    AXC_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(AXC_RUNTIME_ERROR, "device index out of range for the static workspace");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        AXC_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p)
+            return fail(AXC_RUNTIME_ERROR, "hipGetSymbolAddress returned no address for the static workspace");
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return AXC_OK;
+}
 
 // ---- profiling: events around each kernel, on the launch stream ----
 struct ProfEntry {
@@ -649,6 +678,10 @@ int axc_table_create(const uint16_t *host_table, axc_table **out)
         delete tab;
         return fail_hip(e, "table upload");
     }
+    // set-up time is where the static workspace's address on this device is looked up (the lookup may load the
+    // device image); a failure here is reported by axc_conv2d_minmax_static, which looks again
+    void *unused = nullptr;
+    (void)static_scratch(&unused);
     *out = tab;
     return AXC_OK;
 }
@@ -842,6 +875,40 @@ int axc_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc, const
 {
     return run_dense(table, desc, input, filter, nullptr, nullptr, 0, input_min, input_max, filter_min,
                      filter_max, output, nullptr, workspace, workspace_bytes, stream);
+}
+
+int axc_conv2d_static_workspace_limit(size_t *bytes)
+{
+    if (!bytes)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    *bytes = kStaticScratchBytes;
+    return AXC_OK;
+}
+
+int axc_conv2d_minmax_static(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                             const float *filter, float input_min, float input_max, float filter_min,
+                             float filter_max, float *output, void *stream)
+{
+    if (!table || !desc)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    PreparedDense pd;
+    int rc = prepare_dense(desc, &pd);
+    if (rc != AXC_OK)
+        return rc;
+    if (pd.ws.total > kStaticScratchBytes) {
+        char msg[200];
+        snprintf(msg, sizeof(msg), "layer needs %zu bytes of workspace, the static workspace holds %zu: use "
+                 "axc_conv2d_minmax with a caller-owned workspace", pd.ws.total, kStaticScratchBytes);
+        return fail(AXC_INVALID_ARGUMENT, msg);
+    }
+    void *ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc != AXC_OK)
+        return rc;
+    // Every byte of the workspace a launch reads is written by that launch first (codes, sums, packed filter,
+    // partial sums), so what the previous call left in the array needs no clearing.
+    return run_dense(table, desc, input, filter, nullptr, nullptr, 0, input_min, input_max, filter_min, filter_max,
+                     output, nullptr, ws, kStaticScratchBytes, stream);
 }
 
 int axc_conv2d_minmax_acc_i32(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
