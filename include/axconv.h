@@ -199,6 +199,13 @@ int axc_lds_gather_peak(double *lookups_per_second, void *stream);
  * moves at least its 2-byte table entry through that port. */
 int axc_lds_read_peak(double *bytes_per_second, void *stream);
 
+/* Issue rate of the LUT-GEMM's accumulate instructions on this GPU, in lane operations per second over all CUs,
+ * measured with a kernel that contains nothing else, in the LUT-GEMM's occupancy (two wavefronts per SIMD).
+ * The LUT-GEMM spends axc_dense_accumulate_ops_per_lookup() of these operations per table entry, so
+ * rate / ops_per_lookup is the ceiling the vector ALUs put on lookups per second. */
+int axc_valu_issue_peak(double *lane_ops_per_second, void *stream);
+int axc_dense_accumulate_ops_per_lookup(double *ops);
+
 /* Properties of the current device the planner uses. */
 int axc_device_info(int *compute_units, int *lds_bytes_per_workgroup, int *clock_khz);
 

@@ -1019,6 +1019,23 @@ int axc_lds_read_peak(double *bytes_per_second, void *stream)
     return AXC_OK;
 }
 
+int axc_valu_issue_peak(double *lane_ops_per_second, void *stream)
+{
+    if (!lane_ops_per_second)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    *lane_ops_per_second = 0.0;
+    AXC_HIP(run_valu_issue_peak(lane_ops_per_second, kDenseAccumulateMix, static_cast<hipStream_t>(stream)));
+    return AXC_OK;
+}
+
+int axc_dense_accumulate_ops_per_lookup(double *ops)
+{
+    if (!ops)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    *ops = kDenseAccumulateMix == 0 ? 1.0 : 0.75;
+    return AXC_OK;
+}
+
 int axc_device_info(int *compute_units, int *lds_bytes_per_workgroup, int *clock_khz)
 {
     int dev = 0;

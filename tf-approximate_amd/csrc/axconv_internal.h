@@ -22,6 +22,10 @@ constexpr int kDenseWaves = kDenseThreads / 64;
 constexpr int kDenseParkBytes = 16 * 4 * kDenseThreads; // per-thread pixel geometry parked behind the buffers
 constexpr int kBlockThreads = 1024;            // depthwise kernel / LDS probe: 16 wavefronts per CU
 constexpr int kWaves = kBlockThreads / 64;
+// Accumulate instruction mix of the dense kernel's generated phase body (gen_lookup_asm.py emits the same):
+// 0 = one VALU add per table entry (v_add_u32 of a whole dword + v_add_u32_sdwa of its high half);
+// 1 = three per four entries (two dwords of one column pair folded by one v_add3_u32, the high halves by SDWA adds).
+constexpr int kDenseAccumulateMix = 0;
 constexpr uint16_t kNullWeight = 256;          // slot that contributes nothing (padding channel / column)
 
 // Geometry of one dense layer after validation.
@@ -197,5 +201,6 @@ hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float o
                                    uint8_t *wcodes, float *fsum, hipStream_t stream);
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream);
 hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128);
+hipError_t run_valu_issue_peak(double *lane_ops_per_second, int mix, hipStream_t stream);
 
 } // namespace axc

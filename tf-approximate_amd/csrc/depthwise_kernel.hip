@@ -311,6 +311,84 @@ __global__ void __launch_bounds__(kBlockThreads) lds_stream_probe_kernel(uint32_
     out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;
 }
 
+// VALU issue-rate probe: the accumulate instructions of the dense kernel and nothing else, in its own occupancy (one
+// workgroup of 8 wavefronts per CU, two per SIMD).  MIX 0: v_add_u32 / v_add_u32_sdwa alternating (one per
+// table entry); MIX 1: v_add3_u32, v_add_u32_sdwa, v_add_u32_sdwa (three per four entries).  32 independent
+// accumulators, so no instruction waits for the one before it.
+template <int MIX>
+__global__ void __launch_bounds__(kDenseThreads) valu_issue_probe_kernel(uint32_t *out, int iters)
+{
+    uint32_t acc[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+        acc[i] = threadIdx.x + i;
+    uint32_t s0 = threadIdx.x * 2654435761u, s1 = s0 ^ 0x9e3779b9u;
+    for (int it = 0; it < iters; ++it) {
+        // 512 instructions between two branches: the loop overhead stays below half a percent
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+#pragma unroll
+        for (int i = 0; i < 32; i += 4) {
+            if (MIX == 0)
+                asm volatile("v_add_u32 %0, %0, %4\n\t"
+                             "v_add_u32_sdwa %1, %1, %4 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add_u32 %2, %2, %5\n\t"
+                             "v_add_u32_sdwa %3, %3, %5 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
+                             : "+v"(acc[i]), "+v"(acc[i + 1]), "+v"(acc[i + 2]), "+v"(acc[i + 3])
+                             : "v"(s0), "v"(s1));
+            else
+                asm volatile("v_add3_u32 %0, %0, %4, %5\n\t"
+                             "v_add_u32_sdwa %1, %1, %4 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add_u32_sdwa %2, %2, %5 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add3_u32 %3, %3, %5, %4"
+                             : "+v"(acc[i]), "+v"(acc[i + 1]), "+v"(acc[i + 2]), "+v"(acc[i + 3])
+                             : "v"(s0), "v"(s1));
+        }
+    }
+    uint32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+        sum += acc[i];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = sum;
+}
+
+hipError_t run_valu_issue_peak(double *lane_ops_per_second, int mix, hipStream_t stream)
+{
+    int dev = 0, cus = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    uint32_t *out = nullptr;
+    e = hipMalloc(&out, (size_t)cus * kDenseThreads * sizeof(uint32_t));
+    if (e != hipSuccess) return e;
+    auto probe = mix == 0 ? valu_issue_probe_kernel<0> : valu_issue_probe_kernel<1>;
+    // the dense kernel's LDS size: one workgroup per CU
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(probe), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kDenseLdsBytes);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    const int iters = 1500;
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(probe, dim3(cus), dim3(kDenseThreads), kDenseLdsBytes, stream, out, 20);
+        e = hipEventRecord(e0, stream);
+    }
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(probe, dim3(cus), dim3(kDenseThreads), kDenseLdsBytes, stream, out, iters);
+        e = hipEventRecord(e1, stream);
+    }
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e == hipSuccess && ms > 0.0f)
+        *lane_ops_per_second = (double)cus * kDenseThreads * (double)iters * 512.0 / (ms * 1e-3);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    return e;
+}
+
 hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128)
 {
     int dev = 0, cus = 0;

@@ -70,6 +70,10 @@ class ApproxNetwork:
     def conv_count(self):
         return len(self.ops)
 
+    def unfused_layers(self):
+        """With fused_layers: program indices of the convolutions that still run through the calibrated op."""
+        return [i for i, op in self.ops.items() if not isinstance(op, ops.FakeApproxConv2D)]
+
     def forward(self, x, calibrate=False, trace=None):
         """Returns (output tensor, total approximate MACs).  With a list as `trace`, every convolution appends
         (spec, input, filter, (min/max x4), raw output) as host arrays, for layer-by-layer checks."""

@@ -409,6 +409,19 @@ def lds_read_peak():
     return v.value
 
 
+def valu_issue_peak():
+    """Issue rate of the LUT-GEMM's accumulate instruction mix in lane operations per second (measured)."""
+    v = ctypes.c_double()
+    _check(_lib.load().axc_valu_issue_peak(ctypes.byref(v), None))
+    return v.value
+
+
+def dense_accumulate_ops_per_lookup():
+    v = ctypes.c_double()
+    _check(_lib.load().axc_dense_accumulate_ops_per_lookup(ctypes.byref(v)))
+    return v.value
+
+
 def device_info():
     a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     _check(_lib.load().axc_device_info(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
