@@ -116,7 +116,7 @@ def make_table(synth, kind):
             "random": lambda: synth.table_random(13), "exact": synth.table_exact}[kind]()
 
 
-def device_tensors(pkg, xs, fs, codes, seed):
+def device_tensors(pkg, xs, fs, codes, seed, mm=MM):
     """Seeded on-grid input and filter, generated on the device (the float of code q is nudged_min + q * scale)."""
     import torch
     dev = torch.device("cuda:0")
@@ -128,7 +128,7 @@ def device_tensors(pkg, xs, fs, codes, seed):
         qa = torch.randn(xs, generator=g, device=dev).mul_(48.0).abs_().round_().clamp_(0, 255).to(torch.int32)
     qb = torch.randint(0, 256, fs, generator=g, device=dev, dtype=torch.int32)
     out = []
-    for q, lo, hi in ((qa, MM[0], MM[1]), (qb, MM[2], MM[3])):
+    for q, lo, hi in ((qa, mm[0], mm[1]), (qb, mm[2], mm[3])):
         nmin, _, scale, _ = pkg.fake_quant.nudge(lo, hi)
         out.append(q.to(torch.float32).mul_(float(scale)).add_(float(nmin)))
     return out[0], out[1]
@@ -162,12 +162,12 @@ def kernel_times(ops, op, xd, fd, steps):
     return {k: v[0] / max(v[1], 1) for k, v in prof.items()}
 
 
-def sampled_oracle_check(oracle, table, op, xd, fd, strides, depthwise, y, n_samples=12, seed=5):
+def sampled_oracle_check(oracle, table, op, xd, fd, strides, depthwise, y, n_samples=12, seed=5, mm=MM):
     """The oracle's quantize + LUT-GEMM + epilogue on sampled output pixels (corners included) against the int32
     accumulators and the float output of the GPU.  Returns (acc_bit_exact, linf_rel)."""
     import numpy as np
     import torch
-    acc = op.accumulators(xd, fd, *MM)
+    acc = op.accumulators(xd, fd, *mm)
     N, OH, OW, Cout = acc.shape
     _, H, W, C = xd.shape
     KH, KW = fd.shape[0], fd.shape[1]
@@ -191,7 +191,7 @@ def sampled_oracle_check(oracle, table, op, xd, fd, strides, depthwise, y, n_sam
     got_y = y[idx(n_i), idx(np.array([p[1] for p in picks])), idx(np.array([p[2] for p in picks]))].cpu().numpy()
     f = fd.cpu().numpy()
 
-    qp = oracle.quant_props(*MM)
+    qp = oracle.quant_props(*mm)
     f32 = np.float32
     qa = oracle.quantize(vals, qp.in_offset, qp.in_inv_scale)      # taps outside hold 0.0f -> the zero-point code
     qb = oracle.quantize(f, qp.f_offset, qp.f_inv_scale)

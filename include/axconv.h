@@ -8,7 +8,9 @@
  * min/max values are host scalars passed by value, as the reference pins them to host
  * memory (tf2/src/approx_nn_conv_ops.cpp:691-694).  `stream` is a hipStream_t passed as
  * void* (NULL = the default stream).  Launch calls are asynchronous on that stream, allocate
- * nothing and keep no state between calls: the caller owns the workspace.
+ * nothing and keep no state between calls (tile plans are cached by layer shape, which callers cannot observe):
+ * the caller owns the workspace.  A table belongs to the device that was current at its creation; launches with
+ * another device current are refused.
  *
  * Each declaration cites the reference interface (paths under tf2/src/) it replaces.
  */
@@ -122,10 +124,23 @@ int axc_axconv2d_quint8(const axc_table *table, const axc_conv2d_desc *desc, con
  * uint16[65536] in host memory and may be the same buffer. */
 int axc_table_tune_weights(const uint16_t *table, uint16_t *tuned);
 
+/* The two TensorFlow quantization helpers AxQuantizedConv2DOp::Compute calls around the functor
+ * (tf1/axqconv/axqconv.cc:364-367,427-431), as the reference's copy of them defines them
+ * (tf1/axqconv/quantization_utils.h:49-64,114-140): the quint8 code of 0.0f for a float range (offset_input /
+ * offset_filter of axc_axconv2d_quint8), and the float range the qint32 output stands for. */
+int axc_quint8_zero_point(float range_min, float range_max, int32_t *zero_point);
+int axc_qint32_range_for_multiplication(float min_a, float max_a, float min_b, float max_b, float *min_c,
+                                        float *max_c);
+
 /* How the dense kernel would cut this layer on the current device (for tools and tests; the reference has no
  * counterpart, its launch shapes are fixed in cuda/approx_nn_conv_kernels.cu:296-627):
  * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups }. */
 int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6]);
+/* Pins the tile width the planner uses (16, 32 or 64 columns; 0 = its own choice, the default), process-wide, for
+ * tests and timing of the wider-tile kernel variants.  The environment variable AXC_TILE_COLUMNS gives the initial
+ * value and is read once, when the library is loaded.  This is the library's only setting; a workspace query and
+ * the launch it is for must see the same value. */
+int axc_set_tile_columns(int columns);
 int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
 
 /* The op: replaces ApproxConv2DOp::Compute -> LaunchApproxConv2DOp<GPUDevice> and the kernels it

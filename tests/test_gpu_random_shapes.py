@@ -91,11 +91,18 @@ def test_extreme_shapes_vs_oracle(pkg, oracle, case):
 
 
 @pytest.mark.parametrize("columns", [32, 64])
-def test_wider_column_tiles_vs_oracle(pkg, oracle, columns, monkeypatch):
+def test_wider_column_tiles_vs_oracle(pkg, oracle, columns):
     """The tile planner has so far always chosen 16-column tiles; the 32- and 64-column variants of the kernel
     (other accumulator shapes, rotated activation dwords, the untransposed store path for 64) are pinned here by
-    forcing the width through the environment."""
-    monkeypatch.setenv("AXC_TILE_COLUMNS", str(columns))
+    forcing the width through axc_set_tile_columns."""
+    pkg.ops.set_tile_columns(columns)
+    try:
+        _wider_tile_cases(pkg, oracle, columns)
+    finally:
+        pkg.ops.set_tile_columns(0)
+
+
+def _wider_tile_cases(pkg, oracle, columns):
     mm = (-1.0, 1.0, -0.5, 0.5)
     cases = [((2, 24, 24, 16), (3, 3, 16, 64), (1, 1), (1, 1), "SAME"),
              ((1, 17, 19, 8), (1, 1, 8, 48), (2, 2), (1, 1), "SAME"),
@@ -115,3 +122,46 @@ def test_wider_column_tiles_vs_oracle(pkg, oracle, columns, monkeypatch):
         assert rc == 0
         assert np.array_equal(acc, acc_ref), (columns, xs, fs)
         assert refimpl.linf_rel(y, y_ref) <= 1e-5, (columns, xs, fs)
+
+
+def _sweep_case(seed):
+    """Case `seed` of the wider sweep: the random layer above, sometimes with larger images and batches (several
+    tiles, K splits, partial tiles), every fifth case depthwise, every second input off the quantization grid."""
+    rng = np.random.default_rng(50000 + seed)
+    xs, fs, strides, dil, padding, mm = _random_case(rng)
+    if seed % 3 == 0 and fs[2] <= 32:
+        xs = (int(rng.integers(1, 6)), int(rng.integers(max(20, (fs[0] - 1) * dil[0] + 1), 70)),
+              int(rng.integers(max(20, (fs[1] - 1) * dil[1] + 1), 70)), xs[3])
+    dw = seed % 5 == 4
+    if dw:
+        fs = (fs[0], fs[1], fs[2], 1)
+        if seed % 2:
+            fs, dil, strides = (3, 3, fs[2], 1), (1, 1), (int(rng.choice([1, 2])),) * 2
+        if xs[1] < (fs[0] - 1) * dil[0] + 1 or xs[2] < (fs[1] - 1) * dil[1] + 1:
+            return None
+    return xs, fs, strides, dil, padding, mm, dw
+
+
+@pytest.mark.parametrize("block", range(5))
+def test_random_sweep_slice_vs_oracle(pkg, oracle, block):
+    """150 fixed-seed cases of the sweep (30 per test), dense and depthwise, whole outputs against the oracle."""
+    for seed in range(block * 30, block * 30 + 30):
+        case = _sweep_case(seed)
+        if case is None:
+            continue
+        xs, fs, strides, dil, padding, mm, dw = case
+        print("sweep case", seed, xs, fs, strides, dil, padding, "depthwise" if dw else "dense", flush=True)
+        x, f, _, _ = refimpl.grid_case(pkg, xs, fs, mm, seed=seed)
+        if seed % 2:
+            x = (x + np.float32(0.0013)).astype(np.float32)
+        table = pkg.synth.table_random(seed)
+        y, acc = gpu_util.run_op(pkg, table, x, f, mm, strides, padding, dil, depthwise=dw)
+        if dw:
+            rc, y_ref, acc_ref = oracle.depthwise_conv2d(table, x, f, *mm, strides=strides, padding=padding,
+                                                          dilations=dil)
+        else:
+            rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding,
+                                                    dilations=dil, threads=16)
+        assert rc == 0 and acc.shape == acc_ref.shape, (seed, case)
+        assert np.array_equal(acc, acc_ref), (seed, case)
+        assert refimpl.linf_rel(y, y_ref) <= 1e-5, (seed, case)

@@ -231,3 +231,62 @@ def test_table_from_a_c_model(pkg, golden_dir, tmp_path):
         tables.table_from_c_model(str(src), "no_such_function")
     with pytest.raises(ValueError):
         tables.table_from_c_model(str(src), "mul exact")
+
+
+def test_table_tuning_matches_argmin_with_the_tie_rule(ops, oracle, pkg):
+    """axc_table_tune_weights against an independent numpy arg-min (first smallest column, own column wins ties)
+    and against the oracle's restatement of the reference loop."""
+    i = np.arange(256, dtype=np.int64)[:, None]
+    for table in (pkg.synth.table_noisy(7), pkg.synth.table_truncated(4), pkg.synth.table_random(3),
+                  pkg.synth.table_exact()):
+        t = np.asarray(table, np.uint16).reshape(256, 256).astype(np.int64)
+        want = np.empty((256, 256), np.uint16)
+        for w in range(256):
+            err = np.abs(i * w - t).sum(axis=0)             # per candidate column
+            best = int(np.argmin(err))
+            if err[w] == err[best]:
+                best = w
+            want[:, w] = t[:, best]
+        got = ops.tune_table(table).reshape(256, 256)
+        assert np.array_equal(got, want)
+        assert np.array_equal(got.reshape(-1), oracle.table_tune_weights(table))
+    # a tie the own column must win: columns 5 and 9 both exact for weight 9
+    t = pkg.synth.table_exact().reshape(256, 256).copy()
+    t[:, 5] = t[:, 9]
+    assert np.array_equal(ops.tune_table(t).reshape(256, 256)[:, 9], t[:, 9])
+    t2 = pkg.synth.table_exact().reshape(256, 256).copy()
+    t2[:, 9] = 0                                            # weight 9's own column is bad, 5 holds its products
+    t2[:, 5] = np.arange(256) * 9
+    assert np.array_equal(ops.tune_table(t2).reshape(256, 256)[:, 9], t2[:, 5])
+
+
+def test_tf1_zero_point_and_output_range_closed_forms(ops):
+    """FloatToQuantizedUnclamped<quint8>(0, min, max) and QuantizationRangeForMultiplication<quint8, quint8, qint32>
+    (tf1/axqconv/quantization_utils.h:49-64,114-140) on cases the formula fixes by hand."""
+    zp = ops.float_to_quantized_unclamped_quint8
+    assert zp(0.0, 0.0, 1.0) == 0 and zp(0.0, 0.0, 6.0) == 0           # min = 0: code 0
+    assert zp(0.0, -1.0, 1.0) == 128                                    # -1 * 127.5 = -127.5 rounds away from zero
+    assert zp(0.0, -0.5, 1.5) == 64                                     # -0.5 * 127.5 = -63.75
+    assert zp(0.0, -3.0, 0.0) == 255                                    # -3 * 85 = -255
+    assert zp(0.0, 1.0, 3.0) == -128                                    # unclamped: 0 lies below the range, 1 * 127.5
+    assert zp(0.0, 2.0, 2.0) == 0                                       # empty range: lowest code
+    # exhaustive on a grid against exact rational arithmetic
+    from fractions import Fraction
+    rng = np.random.default_rng(4)
+    for _ in range(200):
+        lo, hi = sorted(np.float32(rng.uniform(-8, 8, size=2)))
+        if lo == hi:
+            continue
+        width = Fraction(float(np.float32(hi - lo)))                    # the reference subtracts in float
+        scale = Fraction(256) / (width * Fraction(256, 255))
+        v = Fraction(float(lo)) * scale
+        if abs(v - round(v)) == Fraction(1, 2) or abs((abs(v) % 1) - Fraction(1, 2)) < Fraction(1, 10 ** 6):
+            continue                                                    # stay away from what double rounding decides
+        want = -int(abs(v) + Fraction(1, 2)) * (1 if v >= 0 else -1)
+        assert zp(0.0, float(lo), float(hi)) == want
+    lo, hi = ops.quantization_range_for_multiplication(0.0, 255.0, 0.0, 255.0)
+    assert lo == -2147483648.0 and hi == 2147483648.0                   # one level = 1.0; int32 max rounds up in float
+    lo, hi = ops.quantization_range_for_multiplication(-1.0, 1.0, 0.0, 510.0)
+    level = np.float32(np.float32(2.0) / np.float32(255.0)) * np.float32(2.0)
+    assert np.float32(lo) == np.float32(level * np.float32(-2147483648.0)) and np.float32(hi) == -np.float32(lo)
+    assert ops.quantization_range_for_multiplication(1.0, 1.0, 0.0, 1.0) == (0.0, 0.0)

@@ -83,7 +83,19 @@ def test_reference_test_recipe(oracle, pkg):
     assert refimpl.linf_rel(y, refimpl.torch_conv2d_f64(x, f)) < 1e-6
 
 
-@pytest.mark.parametrize("case", [c for c in CASES if c[4] == (1, 1)][:6])
+# SAME padding with an odd total (even filters, strides that leave one spare row): the im2col form takes
+# pad_before = total / 2 from the windowed-output-size rule, the direct form its own origin
+# ((O - 1) * s + K - I) / 2 (approx_nn_conv_ops_ref.cpp:242-251); the two must pick the same origin.
+ODD_TOTAL_CASES = [
+    ((1, 10, 10, 1), (8, 8, 1, 1), (1, 1), "SAME", (1, 1)),    # total 7: before 3, after 4
+    ((2, 9, 11, 3), (4, 2, 3, 5), (2, 3), "SAME", (1, 1)),     # rows: total 3; cols: total 0 (11 = 3*3 + 2)
+    ((1, 7, 6, 2), (2, 2, 2, 3), (1, 1), "SAME", (1, 1)),      # total 1: before 0, after 1
+    ((1, 8, 8, 2), (4, 4, 2, 3), (2, 2), "SAME", (1, 1)),      # total 2 with an even filter
+    ((1, 5, 5, 1), (2, 3, 1, 2), (2, 2), "SAME", (1, 1)),      # rows total 1, cols total 2
+]
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c[4] == (1, 1)][:6] + ODD_TOTAL_CASES)
 def test_im2col_form_equals_direct_form(oracle, pkg, case):
     """The reference's two statements of the formula (im2col+GEMM vs the direct 7-deep loop) agree."""
     xs, fs, strides, padding, _ = case

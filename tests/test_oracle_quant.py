@@ -87,3 +87,30 @@ def test_fake_quant_lands_on_grid_and_is_idempotent(pkg, oracle):
         # host mirror of Nudge agrees with the oracle's
         hmin, hmax, hscale, hzp = pkg.fake_quant.nudge(vmin, vmax)
         assert (np.float32(nmin), np.float32(nmax), np.float32(scale)) == (hmin, hmax, hscale)
+
+
+def test_fake_quant_ties_clamp_edges_and_one_sided_ranges(pkg):
+    """Fixed vectors worked out by hand from Nudge and the fake-quant formula
+    floor((clamp(x) - nudged_min) / scale + 0.5) * scale + nudged_min, on ranges whose scale is a power of two so
+    that every float operation is exact: ties round half UP (not to even, not away from zero), values at and
+    beyond both nudged ends clamp, and ranges that do not contain zero are nudged until they do."""
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    f32 = np.float32
+    # (0, 255): scale 1, zero point 0, grid = the integers 0..255
+    x = np.array([0.0, 0.49, 0.5, 1.5, 2.5, 3.5, 254.5, 255.0, 255.49, 300.0, -0.3, -7.0], f32)
+    want = np.array([0.0, 0.0, 1.0, 2.0, 3.0, 4.0, 255.0, 255.0, 255.0, 255.0, 0.0, 0.0], f32)
+    assert np.array_equal(fq(x, 0.0, 255.0), want)
+    # (-64, 63.5): scale 0.5, zero point 128, grid = -64 + i/2; ties sit at odd quarters
+    x = np.array([-64.0, -63.75, -63.76, -63.5, -0.25, 0.25, 63.25, 63.5, 63.74, 99.0, -64.2, -1e9], f32)
+    want = np.array([-64.0, -63.5, -64.0, -63.5, 0.0, 0.5, 63.5, 63.5, 63.5, 63.5, -64.0, -64.0], f32)
+    assert np.array_equal(fq(x, -64.0, 63.5), want)
+    # min > 0: (32, 96) has scale 64/255 and a zero point below 0 -> nudged to [0, 255 * scale]
+    nmin, nmax, scale, zp = pkg.fake_quant.nudge(32.0, 96.0)
+    assert zp == 0 and nmin == 0.0 and nmax == f32(f32(255.0) * scale)
+    assert np.array_equal(fq(np.array([-5.0, 0.0, 1000.0], f32), 32.0, 96.0), np.array([0.0, 0.0, nmax], f32))
+    # max < 0: (-96, -32) -> zero point 255, nudged to [-255 * scale, 0]
+    nmin, nmax, scale, zp = pkg.fake_quant.nudge(-96.0, -32.0)
+    assert zp == 255 and nmax == 0.0 and nmin == f32(f32(-255.0) * scale)
+    assert np.array_equal(fq(np.array([-1000.0, 0.0, 5.0], f32), -96.0, -32.0), np.array([nmin, 0.0, 0.0], f32))
+    # min == max == 0: the op's quantization constants are all zero (approx_ops_types.h:142-151) and every value maps to 0
+    assert np.array_equal(fq(np.array([-1.0, 0.0, 2.0], f32), 0.0, 0.0), np.zeros(3, f32))

@@ -55,6 +55,7 @@ SYMBOLS = [
     ("axc_conv2d_geometry", ctypes.c_int, [_desc, ctypes.POINTER(ConvDims)]),
     ("axc_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
     ("axc_conv2d_tile_plan", ctypes.c_int, [_desc, ctypes.POINTER(ctypes.c_int32)]),
+    ("axc_set_tile_columns", ctypes.c_int, [ctypes.c_int]),
     ("axc_depthwise_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
@@ -63,6 +64,8 @@ SYMBOLS = [
     ("axc_fake_approx_conv2d", ctypes.c_int, [_vp, _desc, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
     ("axc_axconv2d_quint8", ctypes.c_int, [_vp, _desc, _vp, _vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp, _sz, _vp]),
     ("axc_table_tune_weights", ctypes.c_int, [_vp, _vp]),
+    ("axc_quint8_zero_point", ctypes.c_int, [_f, _f, ctypes.POINTER(ctypes.c_int32)]),
+    ("axc_qint32_range_for_multiplication", ctypes.c_int, [_f, _f, _f, _f, ctypes.POINTER(_f), ctypes.POINTER(_f)]),
     ("axc_quantize", ctypes.c_int, [_vp, _i64, _f, _f, _vp, _vp]),
     ("axc_conv2d_minmax_acc_i32", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax_acc_i32", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),

@@ -6,11 +6,13 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <map>
 #include <mutex>
 #include <string>
+#include <tuple>
 #include <vector>
 
 using namespace axc;
@@ -140,6 +142,16 @@ void prof_drain_locked(ProfEntry &pe)
         (void)hipEventDestroy(ev.second);
     }
     pe.pending.clear();
+}
+
+// A table lives in the memory of the device that was current when it was created.
+int check_table_device(const axc_table *table)
+{
+    int dev = 0;
+    AXC_HIP(hipGetDevice(&dev));
+    if (dev != table->device)
+        return fail(AXC_INVALID_ARGUMENT, "the truth table was created on another device than the current one");
+    return AXC_OK;
 }
 
 // ---- quantization parameters (approx_ops_types.h:29-49,135-197) ----
@@ -322,18 +334,21 @@ ConvGeom make_geom(const axc_conv2d_dims &dm)
 }
 
 
+// Forced tile width (0 = the planner chooses): set by axc_set_tile_columns; the environment variable
+// AXC_TILE_COLUMNS gives its initial value, read once when the library is loaded.
+std::atomic<int> g_forced_nt{[] {
+    const char *env = std::getenv("AXC_TILE_COLUMNS");
+    const int v = env ? std::atoi(env) : 0;
+    return (v == 16 || v == 32 || v == 64) ? v : 0;
+}()};
+
 // Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
 // Derive cost per fill is constant; lookup cost per fill grows with the wavefront-rows a SIMD carries.
-DensePlan make_plan(const ConvGeom &g, int cus)
+DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt)
 {
     DensePlan best{};
     double best_cost = 1e300;
     const int taps = g.KH * g.KW;
-    // AXC_TILE_COLUMNS=16|32|64 pins the tile width (for tests of the wider tiles and for experiments; the cost
-    // model itself has so far always preferred 16 on this GPU)
-    int forced_nt = 0;
-    if (const char *env = std::getenv("AXC_TILE_COLUMNS"))
-        forced_nt = std::atoi(env);
     for (int nt : {16, 32, 64}) {
         if (forced_nt == 16 || forced_nt == 32 || forced_nt == 64) {
             if (nt != forced_nt)
@@ -390,6 +405,35 @@ DensePlan make_plan(const ConvGeom &g, int cus)
         }
     }
     return best;
+}
+
+// The plan depends on (taps, channel quads, columns, pixels, CUs, forced width) only: looked up instead of
+// recomputed on every workspace query and launch.
+DensePlan make_plan(const ConvGeom &g, int cus)
+{
+    struct Key {
+        int taps, c4, co, cus, forced;
+        int64_t m;
+        bool operator<(const Key &o) const
+        {
+            return std::tie(taps, c4, co, cus, forced, m) < std::tie(o.taps, o.c4, o.co, o.cus, o.forced, o.m);
+        }
+    };
+    static std::mutex mu;
+    static std::map<Key, DensePlan> cache;
+    const Key key{g.KH * g.KW, g.C4, g.Co, cus, g_forced_nt.load(std::memory_order_relaxed), g.M};
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = cache.find(key);
+        if (it != cache.end())
+            return it->second;
+    }
+    const DensePlan plan = compute_plan(g, cus, key.forced);
+    std::lock_guard<std::mutex> lock(mu);
+    if (cache.size() >= 4096)
+        cache.clear();
+    cache[key] = plan;
+    return plan;
 }
 
 inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -453,6 +497,8 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
 {
     if (!table || !desc)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
+    if (int rc_dev = check_table_device(table))
+        return rc_dev;
     if (activation != AXC_ACT_NONE && activation != AXC_ACT_RELU)
         return fail(AXC_INVALID_ARGUMENT, "unknown activation");
     PreparedDense pd;
@@ -579,6 +625,8 @@ int run_depthwise(const axc_table *table, const axc_conv2d_desc *desc, const flo
 {
     if (!table || !desc)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
+    if (int rc_dev = check_table_device(table))
+        return rc_dev;
     axc_conv2d_dims dm;
     int rc = geometry(desc, &dm);
     if (rc != AXC_OK)
@@ -813,27 +861,76 @@ int axc_axconv2d_quint8(const axc_table *table, const axc_conv2d_desc *desc, con
     return AXC_OK;
 }
 
-// AxTune of ApproximateSelector::init (tf1/axqconv/approximate_selector.h:52-85): every weight column w is replaced
-// by the column w2 whose products are closest (sum of absolute errors over all inputs) to the exact i * w.
+// AxTune of ApproximateSelector::init (tf1/axqconv/approximate_selector.h:52-85): weight column w is replaced by
+// the column whose products are closest to exact multiplication by w (sum of absolute errors over all inputs); on a
+// tie the weight's own column wins, otherwise the lowest column index.
+// Here as a 256 x 256 error matrix built column by column, then one arg-min per row.
 int axc_table_tune_weights(const uint16_t *table, uint16_t *tuned)
 {
     if (!table || !tuned)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
-    std::vector<uint16_t> src(table, table + 65536); // table and tuned may alias
-    for (int w = 0; w < 256; ++w) {
-        int wpos = -1, werr = 0;
-        for (int w2 = 0; w2 < 256; ++w2) {
-            int sumerr = 0;
-            for (int i = 0; i < 256; ++i)
-                sumerr += abs(i * w - (int)src[i * 256 + w2]);
-            if (sumerr < werr || (werr == sumerr && w2 == w) || wpos < 0) {
-                werr = sumerr;
-                wpos = w2;
+    // columns of the source table, contiguous: col[c][i] = table[i][c] (table and tuned may be the same buffer)
+    std::vector<int32_t> col((size_t)256 * 256);
+    for (int i = 0; i < 256; ++i)
+        for (int c = 0; c < 256; ++c)
+            col[(size_t)c * 256 + i] = table[(size_t)i * 256 + c];
+    // err[w][c] = sum_i |i * w - col[c][i]|   (at most 256 * 65535, fits int32)
+    std::vector<int32_t> err((size_t)256 * 256);
+    for (int c = 0; c < 256; ++c) {
+        const int32_t *cc = &col[(size_t)c * 256];
+        for (int w = 0; w < 256; ++w) {
+            int32_t e = 0, exact = 0;
+            for (int i = 0; i < 256; ++i, exact += w) {
+                const int32_t d = exact - cc[i];
+                e += d < 0 ? -d : d;
             }
+            err[(size_t)w * 256 + c] = e;
         }
-        for (int i = 0; i < 256; ++i)
-            tuned[i * 256 + w] = src[i * 256 + wpos];
     }
+    for (int w = 0; w < 256; ++w) {
+        const int32_t *ew = &err[(size_t)w * 256];
+        int best = (int)(std::min_element(ew, ew + 256) - ew);   // the first of the smallest
+        if (ew[w] == ew[best])
+            best = w;                                            // the weight's own column wins a tie
+        const int32_t *cb = &col[(size_t)best * 256];
+        for (int i = 0; i < 256; ++i)
+            tuned[(size_t)i * 256 + w] = (uint16_t)cb[i];
+    }
+    return AXC_OK;
+}
+
+// FloatToQuantizedUnclamped<quint8>(0.0f, range_min, range_max) (tf1/axqconv/quantization_utils.h:49-64): the range
+// is widened by 256/255 in double, and the code of 0.0f is minus the rounded (half away from zero) code of range_min.
+int axc_quint8_zero_point(float range_min, float range_max, int32_t *zero_point)
+{
+    if (!zero_point)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    if (range_min == range_max) {
+        *zero_point = 0;
+        return AXC_OK;
+    }
+    const double steps = 256.0;
+    const float width = range_max - range_min;                   // float, as in the reference
+    const double range = (double)width * (steps / (steps - 1.0));
+    const double range_scale = steps / range;
+    *zero_point = (int32_t)(int64_t)(round(0.0 * range_scale) - round((double)range_min * range_scale));
+    return AXC_OK;
+}
+
+// QuantizationRangeForMultiplication<quint8, quint8, qint32> (tf1/axqconv/quantization_utils.h:114-140): one level of
+// the product is one level of a times one level of b, all in float.
+int axc_qint32_range_for_multiplication(float min_a, float max_a, float min_b, float max_b, float *min_c,
+                                        float *max_c)
+{
+    if (!min_c || !max_c)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    volatile float a_level = (max_a - min_a) / (float)(int64_t)255;
+    volatile float b_level = (max_b - min_b) / (float)(int64_t)255;
+    volatile float c_level = a_level * b_level;
+    volatile float lo = c_level * (float)(int64_t)INT32_MIN;
+    volatile float hi = c_level * (float)(int64_t)INT32_MAX;
+    *min_c = lo;
+    *max_c = hi;
     return AXC_OK;
 }
 
@@ -851,6 +948,14 @@ int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6])
     plan[3] = pd.plan.n_col_tiles;
     plan[4] = pd.plan.k_splits;
     plan[5] = pd.plan.grid;
+    return AXC_OK;
+}
+
+int axc_set_tile_columns(int columns)
+{
+    if (columns != 0 && columns != 16 && columns != 32 && columns != 64)
+        return fail(AXC_INVALID_ARGUMENT, "tile columns must be 0 (planner's choice), 16, 32 or 64");
+    g_forced_nt.store(columns, std::memory_order_relaxed);
     return AXC_OK;
 }
 

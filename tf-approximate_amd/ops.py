@@ -233,29 +233,22 @@ class FakeApproxConv2D:
 
 # ---- tf1 AxConv2D (tf1/axqconv/axqconv.cc) ----------------------------------------------------------------------
 def float_to_quantized_unclamped_quint8(value, range_min, range_max):
-    """TensorFlow's FloatToQuantizedUnclamped<quint8> (tensorflow/core/kernels/quantization_utils.h), which the
-    reference calls with value 0 to get the zero points (tf1/axqconv/axqconv.cc:350-353).  Restated from the
-    published algorithm; nothing in the reference pins it (third-party code)."""
-    if range_max == range_min:
-        return 0
-    steps = 256.0
-    range_adjust = steps / (steps - 1.0)
-    rng = (float(range_max) - float(range_min)) * range_adjust
-    scale = steps / rng
-
-    def rnd(v):  # std::round: half away from zero
-        return int(np.floor(abs(v) + 0.5)) * (1 if v >= 0 else -1)
-    return rnd(float(value) * scale) - rnd(float(range_min) * scale)
+    """FloatToQuantizedUnclamped<quint8> for the value 0.0f (tf1/axqconv/quantization_utils.h:49-64): the zero
+    point the reference derives per tensor (tf1/axqconv/axqconv.cc:364-367).  Computed by the library."""
+    if float(value) != 0.0:
+        raise UnimplementedError("only the code of 0.0f is needed by AxConv2D")
+    zp = ctypes.c_int32()
+    _check(_lib.load().axc_quint8_zero_point(float(range_min), float(range_max), ctypes.byref(zp)))
+    return zp.value
 
 
 def quantization_range_for_multiplication(min_a, max_a, min_b, max_b):
-    """TensorFlow's QuantizationRangeForMultiplication<quint8, quint8, qint32> (same header): the float range the
-    qint32 output of AxConv2D stands for (tf1/axqconv/axqconv.cc:427-431).  Third-party, restated."""
-    f32 = np.float32
-    a_one = f32((f32(max_a) - f32(min_a)) / f32(255.0))
-    b_one = f32((f32(max_b) - f32(min_b)) / f32(255.0))
-    c_one = f32(a_one * b_one)
-    return float(f32(c_one * f32(-2147483648.0))), float(f32(c_one * f32(2147483647.0)))
+    """QuantizationRangeForMultiplication<quint8, quint8, qint32> (tf1/axqconv/quantization_utils.h:114-140): the
+    float range the qint32 output of AxConv2D stands for (tf1/axqconv/axqconv.cc:427-431)."""
+    lo, hi = ctypes.c_float(), ctypes.c_float()
+    _check(_lib.load().axc_qint32_range_for_multiplication(float(min_a), float(max_a), float(min_b), float(max_b),
+                                                           ctypes.byref(lo), ctypes.byref(hi)))
+    return lo.value, hi.value
 
 
 def tune_table(table):
@@ -302,6 +295,11 @@ def conv2d_tile_plan(input_shape, filter_shape, strides=(1, 1, 1, 1), padding="S
     _check(lib.axc_conv2d_tile_plan(ctypes.byref(desc), plan))
     keys = ("columns_per_tile", "rows_per_tile", "row_tiles", "column_tiles", "k_splits", "workgroups")
     return dict(zip(keys, [int(v) for v in plan]))
+
+
+def set_tile_columns(columns):
+    """Pins the dense kernel's tile width (16 / 32 / 64 columns; 0 = the planner's choice) for the whole process."""
+    _check(_lib.load().axc_set_tile_columns(int(columns)))
 
 
 _table_cache = {}
