@@ -82,10 +82,28 @@ PROFILED_TRAFFIC = {
 }
 
 
+def measured_copy_bandwidth(mib=512, reps=30):
+    """Bytes per second (read + written) of a plain device-to-device copy: what HBM sustains for a streaming kernel
+    that reads one buffer and writes another, the depthwise kernels' access pattern."""
+    import torch
+    n = mib * (1 << 20) // 4
+    a = torch.ones(n, dtype=torch.float32, device="cuda:0")
+    b = torch.empty_like(a)
+    for _ in range(10):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    return 2.0 * n * 4 * reps / (time.perf_counter() - t0)
+
+
 class Ceilings:
     """The ceilings of the dense kernel, measured once per run."""
 
     def __init__(self, ops):
+        self.copy_bytes = measured_copy_bandwidth()
         self.gather = ops.lds_gather_peak()                     # conflict-free ds_read_u16 lookups/s
         self.port_bytes = max(ops.lds_read_peak(), 1.0)         # streaming ds_read_b128 bytes/s
         self.valu_lane_ops = max(ops.valu_issue_peak(), 1.0)    # accumulate-instruction lane operations/s
@@ -107,7 +125,8 @@ class Ceilings:
                 "valu_ops_per_lookup": self.ops_per_lookup,
                 "valu_glookups_per_s": round(self.valu_lane_ops / self.ops_per_lookup / 1e9, 1),
                 "nominal_gather_glookups_per_s": round(NOMINAL_LDS_LOOKUPS_PER_S / 1e9, 1),
-                "measured_ds_read_u16_glookups_per_s": round(self.gather / 1e9, 1)}
+                "measured_ds_read_u16_glookups_per_s": round(self.gather / 1e9, 1),
+                "hbm_device_copy_gbytes_per_s": round(self.copy_bytes / 1e9, 1)}
 
 
 def make_table(synth, kind):
@@ -252,7 +271,7 @@ def measure_layer(pkg, ops, oracle, ceil, spec, steps=None, preroll_s=0.08):
         nbytes = 4 * (xd.numel() + y.numel()) + 4 * fd.numel() + 131072
         gbps = nbytes / (kernel_ms * 1e-3) / 1e9
         rec.update({"bound": "hbm", "frac": round(gbps / HBM_PEAK_GBPS, 4), "hbm_algorithmic_gbytes_per_s": round(gbps, 1),
-                    "algorithmic_bytes": nbytes})
+                    "frac_of_device_copy": round(gbps * 1e9 / ceil.copy_bytes, 4), "algorithmic_bytes": nbytes})
     else:
         fr, _ = ceil.fractions(lookups / (kernel_ms * 1e-3))
         rec.update(fr)
@@ -407,6 +426,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(hbm_bytes / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "frac_of_device_copy": round(hbm_bytes / (main_ms * 1e-3) / ceil.copy_bytes, 4),
+            "device_copy_gbytes_per_s": round(ceil.copy_bytes / 1e9, 1),
             "traffic": traffic,
             "traffic_source": traffic_source,
             "kernel_ms": round(main_ms, 4),

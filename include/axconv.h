@@ -103,11 +103,16 @@ int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
  * min / max of the input batch and of the kernel (reduce_min / reduce_max, :233-241), fake quantization of both
  * with them (fake_quant_with_min_max_vars, :235,242: here fused into the kernels that read the tensors), the op,
  * then bias_add and the activation of Conv.call (:261).  bias may be null; activation is AXC_ACT_*.
- * Workspace: axc_conv2d_workspace_bytes.  Dense convolutions only. */
+ * Workspace: axc_conv2d_workspace_bytes.  axc_fake_approx_depthwise_conv2d is the same layer call around the
+ * depthwise variant (filter [rows, cols, C, 1], bias one value per channel; workspace:
+ * axc_depthwise_conv2d_workspace_bytes): the Keras layer wraps whichever convolution it is given. */
 enum { AXC_ACT_NONE = 0, AXC_ACT_RELU = 1 };
 int axc_fake_approx_conv2d(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
                            const float *filter, const float *bias, int activation, float *output, void *workspace,
                            size_t workspace_bytes, void *stream);
+int axc_fake_approx_depthwise_conv2d(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                                     const float *filter, const float *bias, int activation, float *output,
+                                     void *workspace, size_t workspace_bytes, void *stream);
 
 /* The tf1 integer op AxConv2D (tf1/axqconv/axqconv.cc:66-94 registration, :113-278 ReferenceAxConvFunctor,
  * :286-441 AxQuantizedConv2DOp): quint8 input and filter codes in, qint32 out,

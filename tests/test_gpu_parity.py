@@ -388,6 +388,43 @@ def test_fake_approx_conv2d_layer_ties_and_clamp_edges(pkg, oracle):
     assert refimpl.linf_rel(y_even, y_ref) > 100 * TOL
 
 
+DW_LAYER = [
+    # x_shape, f_shape, strides, bias, activation, input range
+    ((2, 14, 14, 40), (3, 3, 40, 1), (1, 1), True, "relu", (-1.0, 2.0)),     # ragged channel group
+    ((1, 17, 15, 64), (3, 3, 64, 1), (2, 2), False, None, (0.0, 4.0)),       # zero point 0, stride 2
+    ((2, 9, 9, 5), (3, 3, 5, 1), (1, 1), True, None, (-3.0, 1.0)),
+    ((1, 12, 12, 8), (5, 3, 8, 1), (1, 2), True, "relu", (-1.0, 1.0)),       # the generic kernel
+    ((3, 30, 30, 192), (3, 3, 192, 1), (1, 1), True, "relu", (-2.0, 2.0)),   # six channel groups, several segments
+]
+
+
+@pytest.mark.parametrize("case", DW_LAYER, ids=[str(i) for i in range(len(DW_LAYER))])
+def test_fake_approx_depthwise_layer_vs_composition(pkg, oracle, case):
+    """The depthwise layer entry point against the same composition as the dense one, with the depthwise oracle:
+    numpy min/max, host fake quantization of both tensors, the op per channel, bias_add, ReLU."""
+    xs, fs, strides, use_bias, activation, (lo, hi) = case
+    rng = np.random.default_rng(xs[1] * 5 + xs[3])
+    x = rng.uniform(lo, hi, size=xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * 0.3).astype(np.float32)
+    bias = rng.uniform(-0.5, 0.5, size=fs[2]).astype(np.float32) if use_bias else None
+    table = pkg.synth.table_truncated(2)
+    layer = pkg.FakeApproxConv2D(strides, table, "same", activation=activation, depthwise=True)
+    dev = gpu_util.dev()
+    y = layer(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev),
+              torch.from_numpy(bias).to(dev) if use_bias else None).cpu().numpy()
+    mm = (float(x.min()), float(x.max()), float(w.min()), float(w.max()))
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    rc, y_ref, _ = oracle.depthwise_conv2d(table, fq(x, mm[0], mm[1]), fq(w, mm[2], mm[3]), *mm, strides=strides,
+                                           padding="SAME", dilations=(1, 1))
+    assert rc == 0
+    if use_bias:
+        y_ref = (y_ref + bias).astype(np.float32)
+    if activation == "relu":
+        y_ref = np.maximum(y_ref, 0.0)
+    assert y.shape == y_ref.shape
+    assert refimpl.linf_rel(y, y_ref) <= TOL
+
+
 def test_fake_approx_conv2d_layer_all_zero_input(pkg):
     """min == max == 0 for the input: every quantization constant of that tensor is 0 (approx_ops_types.h:142-151)."""
     dev = gpu_util.dev()

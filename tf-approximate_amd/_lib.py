@@ -62,6 +62,7 @@ SYMBOLS = [
     ("axc_conv2d_static_workspace_limit", ctypes.c_int, [ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax_static", ctypes.c_int, [_vp, _desc, _vp, _vp, _f, _f, _f, _f, _vp, _vp]),
     ("axc_fake_approx_conv2d", ctypes.c_int, [_vp, _desc, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
+    ("axc_fake_approx_depthwise_conv2d", ctypes.c_int, [_vp, _desc, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
     ("axc_axconv2d_quint8", ctypes.c_int, [_vp, _desc, _vp, _vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp, _sz, _vp]),
     ("axc_table_tune_weights", ctypes.c_int, [_vp, _vp]),
     ("axc_quint8_zero_point", ctypes.c_int, [_f, _f, ctypes.POINTER(ctypes.c_int32)]),

@@ -619,14 +619,33 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     return AXC_OK;
 }
 
+struct DepthwiseWorkspace {
+    size_t wcodes_off, fsum_off, layer_off, total;
+};
+
+DepthwiseWorkspace depthwise_workspace(int taps, int C)
+{
+    DepthwiseWorkspace w;
+    size_t off = 0;
+    w.wcodes_off = off; off += align_up((size_t)taps * C);
+    w.fsum_off = off; off += align_up((size_t)C * 4);
+    w.layer_off = off;  // layer entry point: partial (min, max) pairs of both tensors, then the LayerQuant
+    off += align_up((size_t)4 * kMinMaxBlocks * sizeof(float)) + align_up(sizeof(LayerQuant));
+    w.total = off;
+    return w;
+}
+
 int run_depthwise(const axc_table *table, const axc_conv2d_desc *desc, const float *input, const float *filter,
                   float in_min, float in_max, float f_min, float f_max, float *out_f, int32_t *out_i,
-                  void *workspace, size_t workspace_bytes, void *stream_v)
+                  void *workspace, size_t workspace_bytes, void *stream_v, bool layer_mode = false,
+                  const float *bias = nullptr, int activation = AXC_ACT_NONE)
 {
     if (!table || !desc)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
     if (int rc_dev = check_table_device(table))
         return rc_dev;
+    if (activation != AXC_ACT_NONE && activation != AXC_ACT_RELU)
+        return fail(AXC_INVALID_ARGUMENT, "unknown activation");
     axc_conv2d_dims dm;
     int rc = geometry(desc, &dm);
     if (rc != AXC_OK)
@@ -647,19 +666,29 @@ int run_depthwise(const axc_table *table, const axc_conv2d_desc *desc, const flo
                                 stream));
         return AXC_OK;
     }
-    const size_t wcodes_bytes = align_up((size_t)taps * C);
-    const size_t need = wcodes_bytes + align_up((size_t)C * 4);
-    if (workspace_bytes < need || !workspace)
+    const DepthwiseWorkspace dws = depthwise_workspace(taps, C);
+    if (workspace_bytes < dws.total || !workspace)
         return fail(AXC_INVALID_ARGUMENT, "workspace too small (see axc_depthwise_conv2d_workspace_bytes)");
     if (((uintptr_t)workspace & 255) != 0)
         return fail(AXC_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
     axc_quant_props qp;
     axc_quant_props_compute(in_min, in_max, f_min, f_max, &qp);
-    uint8_t *wcodes = static_cast<uint8_t *>(workspace);
-    float *fsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + wcodes_bytes);
+    char *ws = static_cast<char *>(workspace);
+    uint8_t *wcodes = reinterpret_cast<uint8_t *>(ws + dws.wcodes_off);
+    float *fsum = reinterpret_cast<float *>(ws + dws.fsum_off);
+    const TensorQuant tq_in = {qp.input_offset, qp.input_inv_scale, qp.input_scale, 0.0f, 0u, 0u};
+    const TensorQuant tq_f = {qp.filter_offset, qp.filter_inv_scale, qp.filter_scale, 0.0f, 0u, 0u};
+    LayerQuant *lq_dev = nullptr;
+    if (layer_mode) {
+        ProfScope ps("layer_quant", stream);
+        float *partials = reinterpret_cast<float *>(ws + dws.layer_off);
+        lq_dev = reinterpret_cast<LayerQuant *>(ws + dws.layer_off + align_up((size_t)4 * kMinMaxBlocks * sizeof(float)));
+        AXC_HIP(launch_layer_quant(input, (int64_t)dm.batch * dm.input_rows * dm.input_cols * C, filter,
+                                   (int64_t)taps * C, taps, partials, lq_dev, stream));
+    }
     {
         ProfScope ps("depthwise_filter", stream);
-        AXC_HIP(launch_depthwise_filter(filter, taps, C, qp.filter_offset, qp.filter_inv_scale, wcodes, fsum, stream));
+        AXC_HIP(launch_depthwise_filter(filter, taps, C, tq_f, lq_dev, wcodes, fsum, stream));
     }
     DepthwiseParams p;
     p.N = dm.batch; p.H = dm.input_rows; p.W = dm.input_cols; p.C = C;
@@ -669,12 +698,15 @@ int run_depthwise(const axc_table *table, const axc_conv2d_desc *desc, const flo
     p.M = M;
     p.x = input; p.wcodes = wcodes; p.fsum = fsum; p.tableT = table->dev_tableT;
     p.out_f = out_f; p.out_i = out_i;
-    p.in_offset = qp.input_offset; p.in_inv_scale = qp.input_inv_scale;
+    p.in_q = tq_in;
     p.s1xs2 = qp.s1xs2; p.m1 = qp.m1; p.m2 = qp.m2;
     {
         volatile float km = (float)taps * qp.m1xm2;
         p.k_m1xm2 = km;
     }
+    p.lq_dev = lq_dev;
+    p.bias = bias;
+    p.relu = activation == AXC_ACT_RELU ? 1 : 0;
     const int cus = device_cus();
     const int64_t blocks_needed = (M * C + kBlockThreads - 1) / kBlockThreads;
     const int grid = (int)(blocks_needed < cus ? blocks_needed : cus);
@@ -809,6 +841,16 @@ int axc_fake_approx_conv2d(const axc_table *table, const axc_conv2d_desc *desc, 
         return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
     return run_dense(table, desc, input, filter, nullptr, nullptr, 0, 0.0f, 0.0f, 0.0f, 0.0f, output, nullptr, workspace,
                      workspace_bytes, stream, true, bias, activation);
+}
+
+int axc_fake_approx_depthwise_conv2d(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                                     const float *filter, const float *bias, int activation, float *output,
+                                     void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!output)
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    return run_depthwise(table, desc, input, filter, 0.0f, 0.0f, 0.0f, 0.0f, output, nullptr, workspace,
+                         workspace_bytes, stream, true, bias, activation);
 }
 
 // tf1 AxConv2D: filter origin offsets of ReferenceAxConvFunctor (tf1/axqconv/axqconv.cc:153-163), C integer division
@@ -970,7 +1012,7 @@ int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *by
     rc = validate_for_launch(desc, dm, true);
     if (rc != AXC_OK)
         return rc;
-    *bytes = align_up((size_t)dm.filter_rows * dm.filter_cols * dm.in_depth) + align_up((size_t)dm.in_depth * 4);
+    *bytes = depthwise_workspace(dm.filter_rows * dm.filter_cols, dm.in_depth).total;
     return AXC_OK;
 }
 

@@ -109,8 +109,11 @@ struct DepthwiseParams {
     const uint16_t *tableT;
     float *out_f;
     int32_t *out_i;
-    float in_offset, in_inv_scale;
+    TensorQuant in_q;            // quantization of the input (op entry points: from the host scalars)
     float s1xs2, m1, m2, k_m1xm2;
+    const LayerQuant *lq_dev;    // not null (layer entry point): input quantization and epilogue constants from here
+    const float *bias;           // not null: added per channel after the epilogue
+    int relu;                    // 1: max(x, 0) last
 };
 
 // Row permutation of the expanded table: logical activation code a lives in physical row
@@ -197,8 +200,8 @@ hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials,
 hipError_t launch_axconv_correction(const uint8_t *codes, const uint8_t *fcodes, const ConvGeom &g, int offset_input,
                                     int offset_filter, int32_t *asum, int32_t *bsum, int32_t *out, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t *dst, int64_t n, uint32_t value, hipStream_t stream);
-hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
-                                   uint8_t *wcodes, float *fsum, hipStream_t stream);
+hipError_t launch_depthwise_filter(const float *filter, int taps, int C, const TensorQuant &tq,
+                                   const LayerQuant *lq_dev, uint8_t *wcodes, float *fsum, hipStream_t stream);
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream);
 hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128);
 hipError_t run_valu_issue_peak(double *lane_ops_per_second, int mix, hipStream_t stream);

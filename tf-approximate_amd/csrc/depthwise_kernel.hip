@@ -1,11 +1,28 @@
-// Depthwise LUT convolution (channel multiplier 1) and the LDS gather-rate probe.
+// Depthwise LUT convolution (channel multiplier 1) and the LDS / VALU rate probes.
 #include "axconv_internal.h"
+
+#include <type_traits>
 
 namespace axc {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 extern __shared__ __align__(16) unsigned char lds_dw[];
+
+// Quantization of the input as this launch sees it: by value for the op, from the device for the layer entry point.
+__device__ __forceinline__ TensorQuant dw_input_quant(const DepthwiseParams &p) { return p.lq_dev ? p.lq_dev->in : p.in_q; }
+
+struct DwEpilogue {
+    float s1xs2, m1, m2, k_m1xm2;
+};
+__device__ __forceinline__ DwEpilogue dw_epilogue_consts(const DepthwiseParams &p)
+{
+    if (p.lq_dev)   // K of the layer's constants is the dense patch length; depthwise has K = taps
+        return {p.lq_dev->s1xs2, p.lq_dev->m1, p.lq_dev->m2,
+                __fmul_rn((float)(p.KH * p.KW), __fmul_rn(p.lq_dev->m1, p.lq_dev->m2))};
+    return {p.s1xs2, p.m1, p.m2, p.k_m1xm2};
+}
 
 // Every output (pixel, channel) is its own dot product over the KH*KW taps, so there is no weight
 // reuse across lanes to expand: lanes look single entries up in the LDS-resident table,
@@ -25,6 +42,8 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut_kernel(const Dept
     }
     __syncthreads();
     const uint16_t *table = reinterpret_cast<const uint16_t *>(lds_dw);
+    const TensorQuant q = dw_input_quant(p);
+    const DwEpilogue ep = dw_epilogue_consts(p);
 
     const int64_t total = p.M * p.C;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -43,220 +62,274 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut_kernel(const Dept
                 const int ih = ih0 + kh * p.dh, iw = iw0 + kw * p.dw;
                 float v = 0.0f;
                 if ((unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W)
-                    v = p.x[(((int64_t)n * p.H + ih) * p.W + iw) * p.C + c];
+                    v = fake_quant_value(p.x[(((int64_t)n * p.H + ih) * p.W + iw) * p.C + c], q);
                 psum = __fadd_rn(psum, v);
-                const uint32_t a = quantize_code(v, p.in_offset, p.in_inv_scale);
+                const uint32_t a = quantize_code(v, q.offset, q.inv_scale);
                 const uint32_t b = p.wcodes[(int64_t)tap * p.C + c];
                 acc += (int32_t)table[b * 256u + a];
             }
         if (OUT_I32) {
             p.out_i[idx] = acc;
         } else {
-            const float t0 = __fmul_rn((float)acc, p.s1xs2);
-            const float t1 = __fmul_rn(p.m2, psum);
+            const float t0 = __fmul_rn((float)acc, ep.s1xs2);
+            const float t1 = __fmul_rn(ep.m2, psum);
             const float t2 = __fadd_rn(t0, t1);
-            const float t3 = __fmul_rn(p.m1, p.fsum[c]);
+            const float t3 = __fmul_rn(ep.m1, p.fsum[c]);
             const float t4 = __fadd_rn(t2, t3);
-            p.out_f[idx] = __fsub_rn(t4, p.k_m1xm2);
+            float v = __fsub_rn(t4, ep.k_m1xm2);
+            if (p.bias)
+                v = __fadd_rn(v, p.bias[c]);
+            p.out_f[idx] = p.relu ? fmaxf(v, 0.0f) : v;
         }
     }
 }
 
-// 3x3 filters, dilation 1, column stride SW in {1, 2}: a thread owns one channel of a run of consecutive output
-// pixels of one output row and slides the 3x3 window along it.  Every input value is loaded and quantized once
-// per window row instead of once per tap, and the nine filter codes of the channel live in registers as table row
-// offsets.  Loads and stores go through buffer descriptors with 32-bit offsets: a column or row outside the image
-// gets an offset past the end of the buffer and reads 0.0f without a branch, and 0.0f quantizes to the zero-point
-// code, which is what a tap outside the image looks up.  Same results as depthwise_lut_kernel: taps in (kh, kw)
-// order, zeros (code = zero point) outside the image.
+// ---- 3x3 filters, dilation 1, strides 1 or 2 -------------------------------------------------------------------
+// A workgroup serves kDwChannels consecutive channels.  For them it keeps, in LDS, the table row of every one of the
+// 9 x kDwChannels filter codes, transposed to activation-code major, two taps to a dword:
+//     entry a of (tap t, channel c) at byte  a * kDwCodeStride + (t >> 1) * 128 + c * 4 + (t & 1) * 2
+// with kDwCodeStride = 5 * 128 (the tenth tap slot is unused), 160 KiB in all.  A lane is one channel (two bands of
+// output rows per wavefront: lanes 0-31 and 32-63), and a two-byte read serves 32 lanes per pass over 32 banks:
+// channel c only ever touches bank c, whatever the activation codes are.  The byte offset of an activation code is
+// one multiply-add and the tap is an immediate offset of the read.
+//
+// A lane produces a block of R output rows by `len` output columns: it slides a window of (R-1)*S+3 input rows by 3
+// columns along the row, so an input value is loaded, fake-quantized (layer entry point) and turned into its LDS
+// offset once per block instead of once per output row and tap, and rows shared by the R outputs of a column are
+// fetched once.  Both halves of a wavefront walk the same columns, so column offsets are scalars.  Rows outside the
+// image are buffer offsets past the end, which read 0.0f (the value the reference pads with; it quantizes to the
+// zero-point code) and drop stores, without a branch; columns outside the image are a wave-uniform case.
+// Results are those of depthwise_lut_kernel: taps in (kh, kw) order, the patch sum sequential in that order.
+constexpr int kDwChannels = 32;
+constexpr int kDwCodeStride = 5 * kDwChannels * 4;    // bytes between activation codes: five pairs of taps
+constexpr int kDwLdsBytes = 256 * kDwCodeStride;      // 163840
+
 typedef __amdgpu_buffer_rsrc_t dw_rsrc_t;
 __device__ __forceinline__ dw_rsrc_t dw_make_rsrc(const void *base, uint32_t bytes)
 {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
 
-template <int SW, bool OUT_I32>
+template <int S, int R, bool OUT_I32, bool FQ>
 __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const DepthwiseParams p, const int seg_len,
-                                                                          const int nseg)
+                                                                          const int nseg, const int wgs_per_group,
+                                                                          const int group_slots)
 {
+    constexpr int RIN = (R - 1) * S + 3;               // input rows under R output rows
+    constexpr int CARRY = 3 - S;                       // window columns the next output column keeps
     const int tid = threadIdx.x;
-    {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(p.tableT);
-        u32x4 *dst = reinterpret_cast<u32x4 *>(lds_dw);
-#pragma unroll
-        for (int i = 0; i < kTableBytes / 16 / kBlockThreads; ++i)
-            dst[tid + i * kBlockThreads] = src[tid + i * kBlockThreads];
-    }
-    __syncthreads();
-
-    // the launcher has checked that input and output are below 2 GiB, so offsets from 0x70000000 up are outside
-    constexpr uint32_t kOutside = 0x70000000u;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cl = lane & (kDwChannels - 1), half = lane >> 5;
+    const int slot = (int)blockIdx.x / wgs_per_group, member = (int)blockIdx.x - slot * wgs_per_group;
+    if (slot >= group_slots)
+        return;
+    TensorQuant q = dw_input_quant(p);
+    q.fq = FQ ? 1u : 0u;                                // known at compile time: no branch per value
+    const DwEpilogue ep = dw_epilogue_consts(p);
     const uint32_t x_bytes = (uint32_t)((int64_t)p.N * p.H * p.W * p.C * 4);
     const uint32_t o_bytes = (uint32_t)(p.M * p.C * 4);
     const dw_rsrc_t x_rsrc = dw_make_rsrc(p.x, x_bytes);
     const dw_rsrc_t o_rsrc = dw_make_rsrc(OUT_I32 ? static_cast<const void *>(p.out_i) : static_cast<const void *>(p.out_f), o_bytes);
-    const uint32_t col_bytes = (uint32_t)p.C * 4u;           // bytes between neighbouring pixels of a row
+    const dw_rsrc_t t_rsrc = dw_make_rsrc(p.tableT, (uint32_t)kTableAllocBytes);
+    const uint32_t col_bytes = (uint32_t)p.C * 4u;
+    const int band_pairs = (p.OH + 2 * R - 1) / (2 * R);
+    // a task = (image, pair of bands of R output rows, column segment), segment fastest; the halves of a wavefront
+    // take the two bands of a pair
+    const int tasks = p.N * band_pairs * nseg;
+    const int ngroups = (p.C + kDwChannels - 1) / kDwChannels;
+    // the members of a group take contiguous runs of its tasks: neighbouring bands, which share input rows, stay in
+    // one workgroup (and so in one L2)
+    const int run_first = (int)((int64_t)tasks * member / wgs_per_group);
+    const int run_end = (int)((int64_t)tasks * (member + 1) / wgs_per_group);
 
-    const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;   // (output row segment, channel), channel fastest
-    // Neighbouring output rows read the same input rows.  Workgroups go to the 8 XCDs round-robin and every XCD
-    // has its own L2, so each XCD gets one contiguous band of output rows (whole rows): an input row is then
-    // fetched from memory by one L2 instead of by up to three.
-    const int64_t per_row = (int64_t)nseg * p.C;
-    const int64_t rows_total = (int64_t)p.N * p.OH;
-    int64_t last = items, stride = (int64_t)gridDim.x * blockDim.x;
-    int64_t start = (int64_t)blockIdx.x * blockDim.x + tid;
-    if ((gridDim.x & 7) == 0) {
-        const int xcd = blockIdx.x & 7;
-        const int64_t rows_per_xcd = (rows_total + 7) / 8;
-        const int64_t first = rows_per_xcd * xcd * per_row;
-        last = rows_per_xcd * (xcd + 1) * per_row;
-        last = last < items ? last : items;
-        stride = (int64_t)(gridDim.x >> 3) * blockDim.x;
-        start = first + (int64_t)(blockIdx.x >> 3) * blockDim.x + tid;
-    }
-    constexpr int U = 4;                 // outputs per group
-    constexpr int NEW = U * SW;          // columns that enter the window per group
-    constexpr int CARRY = 3 - SW;        // columns the next group shares with this one
-    for (int64_t item = start; item < last; item += stride) {
-        // items < 2^31 here (the output is below 2 GiB): 32-bit divisions, a fraction of the cost of 64-bit ones
-        const uint32_t it32 = (uint32_t)item;
-        const uint32_t rs = it32 / (uint32_t)p.C;
-        const int c = (int)(it32 - rs * (uint32_t)p.C);
-        const uint32_t row = rs / (uint32_t)nseg;              // n * OH + oh
-        const int seg = (int)(rs - row * (uint32_t)nseg);
-        const int n = (int)(row / (uint32_t)p.OH);
-        const int oh = (int)(row - (uint32_t)n * (uint32_t)p.OH);
-        const int ow0 = seg * seg_len;
-        const int len = (ow0 + seg_len < p.OW ? ow0 + seg_len : p.OW) - ow0;
-        const int ih0 = oh * p.sh - p.ph;
-
-        uint32_t wrow[9];                                      // byte offset of the table row of each tap's filter code
+    for (int group = slot; group < ngroups; group += group_slots) {
+        const int chan = group * kDwChannels + cl;
+        const bool live = chan < p.C;
+        __syncthreads();                                // every wavefront is done with the previous group's rows
+        // ---- stage the 9 x 32 table rows, transposed: a lane takes 8 activation codes (16 bytes of a row) of one
+        // channel for a pair of taps and writes one dword (both taps' entries) per code
+        for (int item = tid; item < 5 * kDwChannels * 32; item += kBlockThreads) {
+            const int c = item & 31, piece = (item >> 5) & 31, tp = item >> 10;
+            const int ch = group * kDwChannels + c;
+            const uint32_t code0 = ch < p.C ? p.wcodes[(2 * tp) * p.C + ch] : kNullWeight;
+            const uint32_t code1 = (ch < p.C && 2 * tp + 1 < 9) ? p.wcodes[(2 * tp + 1) * p.C + ch] : kNullWeight;
+            const u32x4 v0 = __builtin_amdgcn_raw_buffer_load_b128(t_rsrc, (int)(code0 * 512u + (uint32_t)piece * 16u), 0, 0);
+            const u32x4 v1 = __builtin_amdgcn_raw_buffer_load_b128(t_rsrc, (int)(code1 * 512u + (uint32_t)piece * 16u), 0, 0);
+            unsigned char *dst = lds_dw + (8 * piece) * kDwCodeStride + tp * 128 + c * 4;
 #pragma unroll
-        for (int t = 0; t < 9; ++t)
-            wrow[t] = (uint32_t)p.wcodes[t * p.C + c] * 512u;
-        const float t3 = OUT_I32 ? 0.0f : __fmul_rn(p.m1, p.fsum[c]);
-        uint32_t rowbase[3];                                   // byte offset of (n, ih, 0, c); outside for a row that is
-#pragma unroll
-        for (int kh = 0; kh < 3; ++kh) {
-            const int ih = ih0 + kh;
-            rowbase[kh] = (unsigned)ih < (unsigned)p.H
-                              ? (uint32_t)((((int64_t)n * p.H + ih) * p.W * p.C + c) * 4)
-                              : 0x80000000u;
-        }
-        const int iw0 = ow0 * SW - p.pw;                       // input column under tap kw = 0 of the first output
-        auto col_off = [&](int iw) {                           // byte offset of column iw inside a row; outside if none
-            return (unsigned)iw < (unsigned)p.W ? (uint32_t)iw * col_bytes : kOutside;
-        };
-        auto load = [&](int kh, uint32_t coff) {
-            return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(rowbase[kh] + coff), 0, 0));
-        };
-        float cv[3][CARRY + NEW];                              // window columns of the group: values ...
-        uint32_t ca[3][CARRY + NEW];                           // ... and activation codes * 2 (byte offset in a table row)
-#pragma unroll
-        for (int t = 0; t < CARRY; ++t) {
-            const uint32_t coff = col_off(iw0 + t);
-#pragma unroll
-            for (int kh = 0; kh < 3; ++kh) {
-                cv[kh][t] = load(kh, coff);
-                ca[kh][t] = quantize_code(cv[kh][t], p.in_offset, p.in_inv_scale) * 2u;
+            for (int e = 0; e < 4; ++e) {
+                *reinterpret_cast<uint32_t *>(dst + (2 * e) * kDwCodeStride) = (v0[e] & 0xffffu) | (v1[e] << 16);
+                *reinterpret_cast<uint32_t *>(dst + (2 * e + 1) * kDwCodeStride) = (v0[e] >> 16) | (v1[e] & 0xffff0000u);
             }
         }
-        // the columns that enter the window with the next group are loaded one group ahead
-        float pf[3][NEW];
-        auto prefetch = [&](int jfirst) {                      // new columns of outputs jfirst .. jfirst + U - 1
-#pragma unroll
-            for (int t = 0; t < NEW; ++t) {
-                const uint32_t coff = col_off(iw0 + jfirst * SW + CARRY + t);
-#pragma unroll
-                for (int kh = 0; kh < 3; ++kh)
-                    pf[kh][t] = load(kh, coff);
-            }
+        __syncthreads();
+
+        const float t3 = (!OUT_I32 && live) ? __fmul_rn(ep.m1, p.fsum[chan]) : 0.0f;
+        const float bias = (!OUT_I32 && p.bias && live) ? p.bias[chan] : 0.0f;
+        const uint32_t lane_off = (uint32_t)cl * 4u;
+        // value -> (fake-quantized value, byte offset of its code's entries)
+        auto convert = [&](float raw, float &val, uint32_t &off) {
+            val = fake_quant_value(raw, q);
+            off = quantize_code(val, q.offset, q.inv_scale) * (uint32_t)kDwCodeStride + lane_off;
         };
-        prefetch(0);
-        uint32_t o_off = (uint32_t)((((int64_t)row * p.OW + ow0) * p.C + c) * 4);
-        for (int j0 = 0; j0 < len; j0 += U) {
+
+        for (int task = run_first + wave; task < run_end; task += kWaves) {
+            const int seg = task % nseg, nb = task / nseg;
+            const int bp = nb % band_pairs, n = nb / band_pairs;
+            const int oh0 = (2 * bp + half) * R, ow0 = seg * seg_len;
+            const int len = (ow0 + seg_len < p.OW ? ow0 + seg_len : p.OW) - ow0;   // wave-uniform
+            const int ih0 = oh0 * S - p.ph, iw0 = ow0 * S - p.pw;
+            uint32_t rowoff[RIN];
 #pragma unroll
-            for (int kh = 0; kh < 3; ++kh)
+            for (int r = 0; r < RIN; ++r) {
+                const int ih = ih0 + r;
+                rowoff[r] = (live && (unsigned)ih < (unsigned)p.H)
+                                ? (uint32_t)((((int64_t)n * p.H + ih) * p.W * p.C + chan) * 4)
+                                : 0x80000000u;
+            }
+            // column iw of every window row, or zeros when the column is outside the image (iw is wave-uniform)
+            auto load_col = [&](int iw, float (&dst)[RIN]) {
+                if ((unsigned)iw < (unsigned)p.W) {
+                    const uint32_t coff = (uint32_t)iw * col_bytes;
 #pragma unroll
-                for (int t = 0; t < NEW; ++t) {
-                    cv[kh][CARRY + t] = pf[kh][t];
-                    ca[kh][CARRY + t] = quantize_code(pf[kh][t], p.in_offset, p.in_inv_scale) * 2u;
-                }
-            if (j0 + U < len)
-                prefetch(j0 + U);
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (j0 + u >= len)
-                    break;
-                int32_t acc = 0;
-                float psum = 0.0f;
-#pragma unroll
-                for (int kh = 0; kh < 3; ++kh)
-#pragma unroll
-                    for (int kw = 0; kw < 3; ++kw) {
-                        psum = __fadd_rn(psum, cv[kh][u * SW + kw]);
-                        acc += (int32_t)*reinterpret_cast<const uint16_t *>(lds_dw + wrow[kh * 3 + kw] + ca[kh][u * SW + kw]);
-                    }
-                uint32_t outw;
-                if (OUT_I32) {
-                    outw = (uint32_t)acc;
+                    for (int r = 0; r < RIN; ++r)
+                        dst[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)rowoff[r], (int)coff, 0));
                 } else {
-                    const float t0 = __fmul_rn((float)acc, p.s1xs2);
-                    const float t1 = __fmul_rn(p.m2, psum);
-                    const float t2 = __fadd_rn(t0, t1);
-                    const float t4 = __fadd_rn(t2, t3);
-                    outw = __float_as_uint(__fsub_rn(t4, p.k_m1xm2));
+#pragma unroll
+                    for (int r = 0; r < RIN; ++r)
+                        dst[r] = 0.0f;
                 }
-                __builtin_amdgcn_raw_buffer_store_b32(outw, o_rsrc, (int)o_off, 0, 2); // nt: streamed past the caches, which
-                                                                                    // the input rows three output rows share need
-                o_off += col_bytes;
+            };
+            uint32_t ooff[R];                           // byte offset of (n, oh0 + rr, 0, chan) in the output
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr)
+                ooff[rr] = (live && oh0 + rr < p.OH)
+                               ? (uint32_t)((((int64_t)(n * p.OH + oh0 + rr) * p.OW) * p.C + chan) * 4)
+                               : 0x80000000u;
+
+            float val[RIN][3];
+            uint32_t off[RIN][3];
+            float pf[S][RIN];
+            // window of output column 0: physical slot of window column t at output column k is (S*k + t) % 3
+            {
+                float first[3][RIN];
+#pragma unroll
+                for (int t = 0; t < 3; ++t)
+                    load_col(iw0 + t, first[t]);
+#pragma unroll
+                for (int t = 0; t < 3; ++t)
+#pragma unroll
+                    for (int r = 0; r < RIN; ++r)
+                        convert(first[t][r], val[r][t], off[r][t]);
             }
+            auto step = [&](const int k, auto phase_tag) {
+                constexpr int PH = decltype(phase_tag)::value;   // k % 3
+                const bool more = k + 1 < len;
+                if (more) {                                // the columns that enter with output column k + 1
 #pragma unroll
-            for (int kh = 0; kh < 3; ++kh)
-#pragma unroll
-                for (int t = 0; t < CARRY; ++t) {
-                    cv[kh][t] = cv[kh][NEW + t];
-                    ca[kh][t] = ca[kh][NEW + t];
+                    for (int s = 0; s < S; ++s)
+                        load_col(iw0 + (k + 1) * S + CARRY + s, pf[s]);
                 }
+                const uint32_t ocol = (uint32_t)(ow0 + k) * col_bytes;
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    uint32_t e[9];
+                    float psum = 0.0f;
+#pragma unroll
+                    for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+                        for (int kw = 0; kw < 3; ++kw) {
+                            const int ps = (S * PH + kw) % 3;
+                            psum = __fadd_rn(psum, val[rr * S + kh][ps]);
+                            e[kh * 3 + kw] = *reinterpret_cast<const uint16_t *>(lds_dw + off[rr * S + kh][ps] + ((kh * 3 + kw) >> 1) * 128 + ((kh * 3 + kw) & 1) * 2);
+                        }
+                    const uint32_t acc = ((e[0] + e[1] + e[2]) + (e[3] + e[4] + e[5])) + (e[6] + e[7] + e[8]);
+                    uint32_t outw;
+                    if (OUT_I32) {
+                        outw = acc;
+                    } else {
+                        const float t0 = __fmul_rn((float)(int32_t)acc, ep.s1xs2);
+                        const float t1 = __fmul_rn(ep.m2, psum);
+                        const float t2 = __fadd_rn(t0, t1);
+                        const float t4 = __fadd_rn(t2, t3);
+                        float v = __fsub_rn(t4, ep.k_m1xm2);
+                        if (p.bias)
+                            v = __fadd_rn(v, bias);
+                        outw = __float_as_uint(p.relu ? fmaxf(v, 0.0f) : v);
+                    }
+                    // streamed past the caches, which the input rows neighbouring bands share need
+                    __builtin_amdgcn_raw_buffer_store_b32(outw, o_rsrc, (int)ooff[rr], (int)ocol, 2);
+                }
+                if (more) {
+#pragma unroll
+                    for (int s = 0; s < S; ++s) {
+                        const int ps = (S * (PH + 1) + CARRY + s) % 3;
+#pragma unroll
+                        for (int r = 0; r < RIN; ++r)
+                            convert(pf[s][r], val[r][ps], off[r][ps]);
+                    }
+                }
+            };
+            for (int k = 0; k < len; k += 3) {
+                step(k, std::integral_constant<int, 0>());
+                if (k + 1 < len)
+                    step(k + 1, std::integral_constant<int, 1>());
+                if (k + 2 < len)
+                    step(k + 2, std::integral_constant<int, 2>());
+            }
         }
     }
 }
 
 template <typename Kernel, typename... Args>
-static hipError_t launch_with_table_lds(Kernel kernel, int grid, hipStream_t stream, Args... args)
+static hipError_t launch_with_lds(Kernel kernel, int grid, int lds_bytes, hipStream_t stream, Args... args)
 {
-    const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(kernel), kTableBytes);
+    const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(kernel), lds_bytes);
     if (e != hipSuccess)
         return e;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBlockThreads), kTableBytes, stream, args...);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBlockThreads), lds_bytes, stream, args...);
     return hipGetLastError();
 }
 
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream)
 {
-    // the sliding kernel addresses input and output with 32-bit byte offsets and keeps the top of that range free
-    const bool sliding = p.KH == 3 && p.KW == 3 && p.dh == 1 && p.dw == 1 && (p.sw == 1 || p.sw == 2) &&
-                         (int64_t)p.N * p.H * p.W * p.C * 4 < 0x70000000ll && p.M * p.C * 4 < 0x70000000ll;
-    if (sliding) {
-        // runs of at most 32 (stride 2: 16) output pixels per thread: enough items to balance the CUs, few window
-        // restarts, and the rows in flight on an XCD at one time still fit its L2
-        const int run = p.sw == 1 ? 32 : 16;
-        const int nseg = (p.OW + run - 1) / run;
-        const int seg_len = (p.OW + nseg - 1) / nseg;
+    // the 3x3 kernel addresses input and output with 32-bit byte offsets and keeps the top of that range free
+    const bool banked = p.KH == 3 && p.KW == 3 && p.dh == 1 && p.dw == 1 && p.sh == p.sw && (p.sw == 1 || p.sw == 2) &&
+                        (int64_t)p.N * p.H * p.W * p.C * 4 < 0x7fffffffll && p.M * p.C * 4 < 0x7fffffffll;
+    if (banked) {
         const int cus = device_cus();
-        const int64_t items = (int64_t)p.N * p.OH * nseg * p.C;
-        const int64_t blocks = (items + kBlockThreads - 1) / kBlockThreads;
-        int g3 = (int)(blocks < cus ? blocks : cus);
-        if (g3 >= 64)
-            g3 &= ~7;   // a multiple of 8 workgroups: the kernel then keeps bands of output rows on one XCD each
-        if (p.sw == 1)
-            return out_i32 ? launch_with_table_lds(depthwise_lut3x3_kernel<1, true>, g3, stream, p, seg_len, nseg)
-                           : launch_with_table_lds(depthwise_lut3x3_kernel<1, false>, g3, stream, p, seg_len, nseg);
-        return out_i32 ? launch_with_table_lds(depthwise_lut3x3_kernel<2, true>, g3, stream, p, seg_len, nseg)
-                       : launch_with_table_lds(depthwise_lut3x3_kernel<2, false>, g3, stream, p, seg_len, nseg);
+        const int R = p.sw == 1 ? 4 : 2;
+        const int ngroups = (p.C + kDwChannels - 1) / kDwChannels;
+        // Workgroups per channel group, and channel groups served at a time: every group gets the same number of
+        // workgroups so that all finish together.
+        int wgs_per_group = cus / ngroups;
+        int group_slots = ngroups;
+        if (wgs_per_group < 1) {
+            wgs_per_group = 1;
+            group_slots = cus;
+        }
+        const int band_pairs = (p.OH + 2 * R - 1) / (2 * R);
+        // column segments: enough tasks that every wavefront of a group's workgroups gets several, few window restarts
+        const int64_t waves = (int64_t)wgs_per_group * kWaves;
+        int nseg = 1;
+        while (nseg < p.OW && (int64_t)p.N * band_pairs * nseg < 5 * waves && (p.OW + nseg) / (nseg + 1) >= 8)
+            ++nseg;
+        const int seg_len = (p.OW + nseg - 1) / nseg;
+        nseg = (p.OW + seg_len - 1) / seg_len;
+        const int g3 = wgs_per_group * group_slots;
+#define AXC_DW_LAUNCH(S_, R_)                                                                                        \
+    (out_i32 ? launch_with_lds(depthwise_lut3x3_kernel<S_, R_, true, false>, g3, kDwLdsBytes, stream, p, seg_len,    \
+                               nseg, wgs_per_group, group_slots)                                                     \
+     : p.lq_dev ? launch_with_lds(depthwise_lut3x3_kernel<S_, R_, false, true>, g3, kDwLdsBytes, stream, p, seg_len, \
+                                  nseg, wgs_per_group, group_slots)                                                  \
+                : launch_with_lds(depthwise_lut3x3_kernel<S_, R_, false, false>, g3, kDwLdsBytes, stream, p,         \
+                                  seg_len, nseg, wgs_per_group, group_slots))
+        return p.sw == 1 ? AXC_DW_LAUNCH(1, 4) : AXC_DW_LAUNCH(2, 2);
+#undef AXC_DW_LAUNCH
     }
-    return out_i32 ? launch_with_table_lds(depthwise_lut_kernel<true>, grid, stream, p)
-                   : launch_with_table_lds(depthwise_lut_kernel<false>, grid, stream, p);
+    return out_i32 ? launch_with_lds(depthwise_lut_kernel<true>, grid, kTableBytes, stream, p)
+                   : launch_with_lds(depthwise_lut_kernel<false>, grid, kTableBytes, stream, p);
 }
 
 // ---- LDS gather-rate probe: conflict-free ds_read_u16, 16 wavefronts per CU ------------------

@@ -597,18 +597,20 @@ __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restr
 
 // Depthwise filter pre-pass: codes [taps][C] and per-channel sums (taps ascending).
 __global__ void __launch_bounds__(256) depthwise_filter_kernel(const float *__restrict__ filter, int taps, int C,
-                                                                float offset, float inv_scale,
+                                                                const TensorQuant tq,
+                                                                const LayerQuant *__restrict__ lq_dev,
                                                                 uint8_t *__restrict__ wcodes,
                                                                 float *__restrict__ fsum)
 {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= C)
         return;
+    const TensorQuant q = lq_dev ? lq_dev->flt : tq;
     float s = 0.0f;
     for (int t = 0; t < taps; ++t) {
-        const float v = filter[(int64_t)t * C + c];
+        const float v = fake_quant_value(filter[(int64_t)t * C + c], q);
         s = __fadd_rn(s, v);
-        wcodes[(int64_t)t * C + c] = (uint8_t)quantize_code(v, offset, inv_scale);
+        wcodes[(int64_t)t * C + c] = (uint8_t)quantize_code(v, q.offset, q.inv_scale);
     }
     fsum[c] = s;
 }
@@ -1061,11 +1063,11 @@ hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float i
     return hipGetLastError();
 }
 
-hipError_t launch_depthwise_filter(const float *filter, int taps, int C, float offset, float inv_scale,
-                                   uint8_t *wcodes, float *fsum, hipStream_t stream)
+hipError_t launch_depthwise_filter(const float *filter, int taps, int C, const TensorQuant &tq,
+                                   const LayerQuant *lq_dev, uint8_t *wcodes, float *fsum, hipStream_t stream)
 {
     hipLaunchKernelGGL(depthwise_filter_kernel, dim3(blocks_for(C, 256)), dim3(256), 0, stream, filter, taps, C,
-                       offset, inv_scale, wcodes, fsum);
+                       tq, lq_dev, wcodes, fsum);
     return hipGetLastError();
 }
 

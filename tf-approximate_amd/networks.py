@@ -44,7 +44,7 @@ class ApproxNetwork:
     ("conv", dst, src, ConvSpec) | ("add_relu", dst, a, b) | ("maxpool", dst, src)"""
 
     def __init__(self, program, input_shape, table, seed=0, device="cuda:0", fused_layers=False):
-        """fused_layers: run every dense convolution through the layer entry point (min/max of each batch and
+        """fused_layers: run every convolution, dense or depthwise, through the layer entry point (min/max of each batch and
         fake quantization computed on the device, ReLU fused), as the reference's Keras layer does per call;
         otherwise ranges come from a calibration pass and the plain op runs."""
         self.fused_layers = fused_layers
@@ -60,9 +60,10 @@ class ApproxNetwork:
             spec = step[3]
             w = _he_normal(rng, spec.filter_shape())
             self.weights[i] = torch.from_numpy(w).to(self.device)
-            if fused_layers and not spec.depthwise:
+            if fused_layers:
                 self.ops[i] = ops.FakeApproxConv2D((spec.stride, spec.stride), self.table, "SAME",
-                                                   activation="relu" if spec.relu else None)
+                                                   activation="relu" if spec.relu else None,
+                                                   depthwise=spec.depthwise)
             else:
                 self.ops[i] = ops.ApproxConv2DWithMinMaxVars([1, spec.stride, spec.stride, 1], 8, self.table, "SAME",
                                                              depthwise=spec.depthwise)
@@ -84,7 +85,7 @@ class ApproxNetwork:
             if kind == "conv":
                 src, spec = t[step[2]], step[3]
                 w = self.weights[i]
-                if self.fused_layers and not spec.depthwise:
+                if self.fused_layers:
                     y = self.ops[i](src, w)
                     if trace is not None:
                         trace.append((spec, src.cpu().numpy(), w.cpu().numpy(), None, y.cpu().numpy()))

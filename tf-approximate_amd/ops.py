@@ -202,11 +202,14 @@ class FakeApproxConv2D:
     tf2/python/keras/layers/fake_approx_convolutional.py:223-261) as one device-side call: min/max of the batch
     and of the kernel, fake quantization of both, the op, bias_add, activation.  No host synchronisation."""
 
-    def __init__(self, strides, mul_map_file, padding="SAME", dilation_rate=(1, 1), activation=None, num_bits=8):
+    def __init__(self, strides, mul_map_file, padding="SAME", dilation_rate=(1, 1), activation=None, num_bits=8,
+                 depthwise=False):
+        """depthwise: the layer wraps the depthwise variant (kernel [rows, cols, C, 1], bias one value per channel)."""
         if activation not in (None, "relu"):
             raise UnimplementedError("activation %r: only None and 'relu' are fused" % (activation,))
         self.op = ApproxConv2DWithMinMaxVars([1, strides[0], strides[1], 1], num_bits, mul_map_file, padding.upper(),
-                                             dilations=[1, dilation_rate[0], dilation_rate[1], 1])
+                                             dilations=[1, dilation_rate[0], dilation_rate[1], 1], depthwise=depthwise)
+        self.depthwise = depthwise
         self.activation = 1 if activation == "relu" else 0
 
     def __call__(self, inputs, kernel, bias=None):
@@ -215,16 +218,18 @@ class FakeApproxConv2D:
         kernel = _require_device_f32(kernel, "filter")
         if bias is not None:
             bias = _require_device_f32(bias, "bias")
-            if bias.numel() != kernel.shape[3]:
+            if bias.numel() != (kernel.shape[2] if self.depthwise else kernel.shape[3]):
                 raise InvalidArgumentError("bias must have one value per output channel")
         desc = self.op._desc(inputs, kernel)
         dims = conv2d_geometry(desc)
         nbytes = ctypes.c_size_t()
-        _check(lib.axc_conv2d_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)))
+        ws_fn = lib.axc_depthwise_conv2d_workspace_bytes if self.depthwise else lib.axc_conv2d_workspace_bytes
+        _check(ws_fn(ctypes.byref(desc), ctypes.byref(nbytes)))
         ws = _workspace(inputs.device, nbytes.value)
         out = torch.empty(self.op._out_shape(dims), dtype=torch.float32, device=inputs.device)
+        fn = lib.axc_fake_approx_depthwise_conv2d if self.depthwise else lib.axc_fake_approx_conv2d
         with torch.cuda.device(inputs.device):
-            _check(lib.axc_fake_approx_conv2d(self.op.table.handle, ctypes.byref(desc), inputs.data_ptr(),
+            _check(fn(self.op.table.handle, ctypes.byref(desc), inputs.data_ptr(),
                                               kernel.data_ptr(), bias.data_ptr() if bias is not None else None,
                                               self.activation, out.data_ptr(), ws.data_ptr(), ws.numel(),
                                               _stream_ptr(inputs.device)))
