@@ -77,8 +77,10 @@ LAYERS = [
 PROFILED_TRAFFIC = {
     "conv3x3_b64_56x56x64_to_64_s1_same": (2.000 * 13465.0 * 1024 + 1.000 * 72175.1 * 1024,
                                            "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
-    "dw3x3_b64_112x112x192_s1": (2.000 * 838534 * 1024 + 1.000 * 602112 * 1024,
-                                 "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192_s1.md"),
+    "dw3x3_b64_112x112x192_s1": (2.000 * 342889 * 1024 + 1.000 * 602112 * 1024,
+                                 "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
+    "dw3x3_b64_112x112x192_s2": (2.000 * 321245 * 1024 + 1.000 * 150528 * 1024,
+                                 "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
 }
 
 
