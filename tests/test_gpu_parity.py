@@ -198,7 +198,10 @@ def test_codes_entry_point(pkg, oracle):
     table = pkg.TruthTable(table_np)
     for xs, fs, strides, padding, zp in [((2, 9, 8, 5), (3, 3, 5, 11), (1, 1), "SAME", 17),
                                          ((1, 13, 13, 32), (3, 3, 32, 64), (2, 2), "SAME", 0),
-                                         ((3, 6, 6, 16), (1, 1, 16, 48), (1, 1), "VALID", 255)]:
+                                         ((3, 6, 6, 16), (1, 1, 16, 48), (1, 1), "VALID", 255),
+                                         # strided 1x1 filters: only the pixels they read are gathered and quantized
+                                         ((2, 11, 9, 16), (1, 1, 16, 20), (2, 3), "SAME", 9),
+                                         ((2, 10, 10, 7), (1, 1, 7, 5), (3, 2), "VALID", 200)]:
         qa = rng.integers(0, 256, xs).astype(np.uint8)
         qb = rng.integers(0, 256, fs).astype(np.uint8)
         acc = ops.conv2d_codes_acc_i32(table, torch.from_numpy(qa).to(gpu_util.dev()),
@@ -423,6 +426,25 @@ def test_fake_approx_depthwise_layer_vs_composition(pkg, oracle, case):
         y_ref = np.maximum(y_ref, 0.0)
     assert y.shape == y_ref.shape
     assert refimpl.linf_rel(y, y_ref) <= TOL
+
+
+def test_fake_approx_conv2d_layer_strided_1x1_takes_minmax_of_the_whole_input(pkg, oracle):
+    """A strided 1x1 layer reads a quarter of its input, but the layer's min / max are those of the whole tensor
+    (fake_approx_convolutional.py:233-236): the extremes sit on pixels the filter never touches."""
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1.0, 1.0, size=(2, 8, 8, 16)).astype(np.float32)
+    x[0, 1, 1, 3] = 7.5          # odd row and column: skipped by the stride-2 filter
+    x[1, 3, 5, 0] = -6.0
+    w = (rng.standard_normal((1, 1, 16, 24)) * 0.2).astype(np.float32)
+    table = pkg.synth.table_noisy(3)
+    dev = gpu_util.dev()
+    y = pkg.FakeApproxConv2D((2, 2), table, "same")(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev)).cpu().numpy()
+    mm = (float(x.min()), float(x.max()), float(w.min()), float(w.max()))
+    assert mm[:2] == (-6.0, 7.5)
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    rc, y_ref, _ = oracle.conv2d_fast(table, fq(x, *mm[:2]), fq(w, *mm[2:]), *mm, strides=(2, 2), padding="SAME",
+                                      dilations=(1, 1))
+    assert rc == 0 and y.shape == y_ref.shape and refimpl.linf_rel(y, y_ref) <= TOL
 
 
 def test_fake_approx_conv2d_layer_all_zero_input(pkg):

@@ -439,13 +439,15 @@ DensePlan make_plan(const ConvGeom &g, int cus)
 inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct DenseWorkspace {
-    size_t xq_off, psum_off, wq_off, fsum_off, layer_off, part_off, total;
+    size_t sub_off, xq_off, psum_off, wq_off, fsum_off, layer_off, part_off, total;
 };
 
-DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
+// sub_bytes: room for the pixels a strided 1x1 filter reads, gathered into a dense tensor (see prepare_dense)
+DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan, size_t sub_bytes)
 {
     DenseWorkspace w;
     size_t off = 0;
+    w.sub_off = off; off += align_up(sub_bytes);
     w.xq_off = off; off += align_up(((size_t)g.N * g.H + 1) * g.C4 * g.W * 4); // + the zero-point row
     w.psum_off = off; off += align_up((size_t)g.M * 4); // patch sums: one float per output pixel
     w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
@@ -461,13 +463,20 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan)
 
 struct PreparedDense {
     axc_conv2d_dims dims;
-    ConvGeom g;
+    ConvGeom g;          // what the kernels see
+    ConvGeom g_full;     // the layer as given (differs from g when the input is subsampled first)
+    bool subsample;
     DensePlan plan;
     DenseWorkspace ws;
     bool empty;
 };
 
-int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd)
+// A 1x1 filter with a stride only ever reads every stride-th pixel, and never needs padding: the op equals the 1x1
+// stride-1 op on the subsampled input.  Those pixels are gathered into the workspace first (element_bytes each:
+// floats, or bytes for the codes entry point), and every kernel then sees a dense, unpadded stride-1 layer with a
+// quarter (stride 2) of the pixels to quantize and sum.  allow_subsample = false keeps the layer as given (callers
+// with their own padding origin).
+int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_subsample = true, int element_bytes = 4)
 {
     int rc = geometry(desc, &pd->dims);
     if (rc != AXC_OK)
@@ -475,15 +484,25 @@ int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd)
     rc = validate_for_launch(desc, pd->dims, false);
     if (rc != AXC_OK)
         return rc;
-    pd->g = make_geom(pd->dims);
+    pd->g = pd->g_full = make_geom(pd->dims);
+    pd->subsample = false;
     pd->empty = pd->g.M * pd->g.Co == 0; // approx_nn_conv_ops.cpp:449
     if (pd->empty || pd->g.K == 0) {
         pd->plan = DensePlan{};
         pd->ws = DenseWorkspace{};
         return AXC_OK;
     }
+    size_t sub_bytes = 0;
+    if (allow_subsample && pd->g.KH == 1 && pd->g.KW == 1 && (pd->g.sh > 1 || pd->g.sw > 1) && pd->g.ph == 0 &&
+        pd->g.pw == 0) {
+        pd->subsample = true;
+        pd->g.H = pd->g.OH;
+        pd->g.W = pd->g.OW;
+        pd->g.sh = pd->g.sw = 1;
+        sub_bytes = (size_t)pd->g.M * pd->g.C * element_bytes;
+    }
     pd->plan = make_plan(pd->g, device_cus());
-    pd->ws = dense_workspace(pd->g, pd->plan);
+    pd->ws = dense_workspace(pd->g, pd->plan, sub_bytes);
     return AXC_OK;
 }
 
@@ -501,8 +520,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         return rc_dev;
     if (activation != AXC_ACT_NONE && activation != AXC_ACT_RELU)
         return fail(AXC_INVALID_ARGUMENT, "unknown activation");
+    const bool codes_mode = input_codes != nullptr;
     PreparedDense pd;
-    int rc = prepare_dense(desc, &pd);
+    int rc = prepare_dense(desc, &pd, pad_before_override == nullptr, codes_mode ? 1 : 4);
     if (rc != AXC_OK)
         return rc;
     if (pd.empty)
@@ -511,7 +531,6 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         pd.g.ph = pad_before_override[0];
         pd.g.pw = pad_before_override[1];
     }
-    const bool codes_mode = input_codes != nullptr;
     if ((!codes_mode && (!input || !filter)) || (codes_mode && !filter_codes) || (!out_f && !out_i))
         return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
@@ -550,12 +569,24 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     TensorQuant tq_in = {qp.input_offset, qp.input_inv_scale, qp.input_scale, 0.0f, 0u, zp4};
     TensorQuant tq_f = {qp.filter_offset, qp.filter_inv_scale, qp.filter_scale, 0.0f, 0u, 0u};
     LayerQuant *lq_dev = nullptr;
-    if (layer_mode) {
+    if (layer_mode) { // min / max of the whole input tensor, as the layer computes them, whatever the filter reads
         ProfScope ps("layer_quant", stream);
         float *partials = reinterpret_cast<float *>(ws + pd.ws.layer_off);
         lq_dev = reinterpret_cast<LayerQuant *>(ws + pd.ws.layer_off + align_up((size_t)4 * kMinMaxBlocks * sizeof(float)));
-        AXC_HIP(launch_layer_quant(input, (int64_t)g.N * g.H * g.W * g.C, filter, (int64_t)g.K * g.Co, g.K, partials,
+        const ConvGeom &gf = pd.g_full;
+        AXC_HIP(launch_layer_quant(input, (int64_t)gf.N * gf.H * gf.W * gf.C, filter, (int64_t)g.K * g.Co, g.K, partials,
                                    lq_dev, stream));
+    }
+    if (pd.subsample) {
+        ProfScope ps("subsample", stream);
+        const ConvGeom &gf = pd.g_full;
+        void *sub = ws + pd.ws.sub_off;
+        AXC_HIP(launch_subsample(codes_mode ? static_cast<const void *>(input_codes) : static_cast<const void *>(input),
+                                 codes_mode ? 1 : 4, gf.N, gf.H, gf.W, gf.C, gf.sh, gf.sw, g.H, g.W, sub, stream));
+        if (codes_mode)
+            input_codes = static_cast<const uint8_t *>(sub);
+        else
+            input = static_cast<const float *>(sub);
     }
     bool quantized_by_patch_sums = false, filter_done = false;
     if (out_f && !codes_mode) {
@@ -825,11 +856,16 @@ int axc_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes)
 {
     if (!bytes)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
-    PreparedDense pd;
+    // enough for every entry point that takes this workspace: with and without the subsampled copy a strided 1x1
+    // filter gets, floats or codes
+    PreparedDense pd, pd_plain;
     int rc = prepare_dense(desc, &pd);
     if (rc != AXC_OK)
         return rc;
-    *bytes = pd.ws.total;
+    rc = prepare_dense(desc, &pd_plain, false);
+    if (rc != AXC_OK)
+        return rc;
+    *bytes = pd.ws.total > pd_plain.ws.total ? pd.ws.total : pd_plain.ws.total;
     return AXC_OK;
 }
 
@@ -879,7 +915,7 @@ int axc_axconv2d_quint8(const axc_table *table, const axc_conv2d_desc *desc, con
     if (offset_input < 0 || offset_input > 255) // the reference stores it in a quint8 for taps outside the image (:215)
         return fail(AXC_INVALID_ARGUMENT, "offset_input must be in [0, 255]");
     PreparedDense pd;
-    int rc = prepare_dense(desc, &pd);
+    int rc = prepare_dense(desc, &pd, false);
     if (rc != AXC_OK)
         return rc;
     if (pd.empty)

@@ -187,6 +187,9 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
 hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
                               float *partials, LayerQuant *lq_dev, hipStream_t stream);
 constexpr int kMinMaxBlocks = 2048;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch
+// out[n][oh][ow][:] = in[n][oh * sh][ow * sw][:] for tensors of element_bytes-wide elements (C per pixel)
+hipError_t launch_subsample(const void *in, int element_bytes, int N, int H, int W, int C, int sh, int sw, int OH, int OW,
+                            void *out, hipStream_t stream);
 hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
                                  hipStream_t stream);
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,

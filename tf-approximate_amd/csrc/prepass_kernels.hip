@@ -1023,6 +1023,47 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
     return hipGetLastError();
 }
 
+// Gathers the pixels a strided 1x1 filter reads into a dense tensor: VEC bytes per thread and step, pixel_bytes
+// (a multiple of VEC) per pixel.
+template <typename V>
+__global__ void __launch_bounds__(256) subsample_kernel(const V *__restrict__ in, V *__restrict__ out, int64_t total,
+                                                         int per_pixel, int H, int W, int sh, int sw, int OH, int OW)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t pix = i / per_pixel;
+        const int e = (int)(i - pix * per_pixel);
+        const int ow = (int)(pix % OW);
+        const int64_t r = pix / OW;
+        const int oh = (int)(r % OH);
+        const int64_t n = r / OH;
+        out[i] = in[((n * H + (int64_t)oh * sh) * W + (int64_t)ow * sw) * per_pixel + e];
+    }
+}
+
+hipError_t launch_subsample(const void *in, int element_bytes, int N, int H, int W, int C, int sh, int sw, int OH, int OW,
+                            void *out, hipStream_t stream)
+{
+    const int64_t pixel_bytes = (int64_t)C * element_bytes;
+    const int64_t pixels = (int64_t)N * OH * OW;
+    const bool wide = (pixel_bytes & 15) == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0;
+    const int vec = wide ? 16 : (((pixel_bytes & 3) == 0 && ((uintptr_t)in & 3) == 0) ? 4 : 1);
+    const int64_t total = pixels * (pixel_bytes / vec);
+    int64_t blocks = (total + 255) / 256;
+    blocks = blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks);
+    const int per_pixel = (int)(pixel_bytes / vec);
+    if (vec == 16)
+        hipLaunchKernelGGL(subsample_kernel<float4>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           static_cast<const float4 *>(in), static_cast<float4 *>(out), total, per_pixel, H, W, sh, sw, OH, OW);
+    else if (vec == 4)
+        hipLaunchKernelGGL(subsample_kernel<uint32_t>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           static_cast<const uint32_t *>(in), static_cast<uint32_t *>(out), total, per_pixel, H, W, sh, sw, OH, OW);
+    else
+        hipLaunchKernelGGL(subsample_kernel<uint8_t>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           static_cast<const uint8_t *>(in), static_cast<uint8_t *>(out), total, per_pixel, H, W, sh, sw, OH, OW);
+    return hipGetLastError();
+}
+
 hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
                                  hipStream_t stream)
 {
