@@ -149,22 +149,17 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     const rsrc_t tab_rsrc = make_rsrc(p.tableT, (uint32_t)kTableAllocBytes);
     (void)taps;
 
-    // Tiles in the order (row tile, column tile incl. K split), column tile fastest; a workgroup takes a contiguous
-    // run of them, so that its consecutive tiles mostly share their row tile: same pixels, same parked geometry,
-    // same activations.  Workgroups are handed to the 8 XCDs round-robin, and each XCD has its own L2: the runs
-    // are dealt so that neighbouring runs, which share row tiles too, go to workgroups of one XCD.
-    int run_first, run_count;
-    {
-        const int G = (int)gridDim.x;
-        const int w = (G & 7) == 0 ? ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
-        const int per = ntiles / G, extra = ntiles - per * G;
-        run_first = w * per + (w < extra ? w : extra);
-        run_count = per + (w < extra ? 1 : 0);
-    }
+    // Tiles in the order (row tile, column tile incl. K split), column tile fastest, dealt round-robin: at any time
+    // the workgroups work on neighbouring tiles, i.e. on the column tiles of a few row tiles.  Workgroups are handed
+    // to the 8 XCDs round-robin, and each XCD has its own L2: the deal goes by a workgroup index in which neighbours
+    // sit on one XCD, so the column tiles of a row tile (same activations; outputs in the same memory lines, written
+    // at about the same time) meet in one L2.
+    const int G = (int)gridDim.x;
+    const int wg = (G & 7) == 0 ? ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
     int prev_rt = -1;
     bool rvalid[DenseCfg<NT>::R];    // this lane's pixel exists
     uint32_t nr = 0;                 // pixels of this lane whose wavefront row exists (a prefix; wave-uniform)
-    for (int tile = run_first; tile < run_first + run_count; ++tile) {
+    for (int tile = wg; tile < ntiles; tile += G) {
         const int rt = tile / nct_v;
         int ct = tile - rt * nct_v;
         const int ksi = ct / p.plan.n_col_tiles;           // K split of this tile
