@@ -125,19 +125,35 @@ def test_the_model_notices_a_missing_wait():
 def test_every_accumulator_gets_its_share_of_a_fill(nt):
     """A fill holds 64 / NT input channels for each of NT columns: on the path of a full lane every accumulator of
     every pixel must receive exactly that many table entries, half of the columns from the low halves of the dwords
-    (plain add of the dword) and half from the high halves (SDWA WORD_1)."""
+    (add of whole dwords: one per v_add_u32, two per v_add3_u32) and half from the high halves (SDWA WORD_1), and
+    every landed dword must be used exactly twice: once whole, once for its high half."""
     gen = _generator()
     rows = 2 * (64 // nt)
     path = max(_paths(_instructions(gen.emit(nt, 0))), key=len)
-    adds = {}
+    adds, uses = {}, {}
     for text in path:
-        if text.startswith("v_add_u32"):
-            dst = TOKEN.search(text).group(0)
+        if text.startswith("v_add_u32") or text.startswith("v_add3_u32"):
+            toks = TOKEN.findall(text)
+            dst = toks[0]
             if dst.startswith("%[c"):
-                adds.setdefault(dst, []).append("WORD_1" in text)
+                assert toks[1] == dst                       # accumulates in place
+                sources = toks[2:]
+                assert len(sources) == (2 if text.startswith("v_add3") else 1)
+                high = "WORD_1" in text
+                adds.setdefault(dst, []).extend([high] * len(sources))
+                for src in sources:
+                    uses.setdefault(src, []).append(high)
     assert len(adds) == rows * nt
     for r in range(rows):
         for j in range(nt):
             kinds = adds["%%[c%d_%d]" % (r, j)]
             assert len(kinds) == 64 // nt
             assert all(k == bool(j & 1) for k in kinds)
+    # 32 landing registers, each read whole and for its high half once per pixel
+    assert len(uses) == 32
+    for src, kinds in uses.items():
+        assert sorted(kinds) == [False] * rows + [True] * rows, src
+    if nt < 64:    # three accumulate operations per four entries
+        n_ops = sum(1 for t in path if t.startswith("v_add_u32") or t.startswith("v_add3_u32"))
+        n_acc = sum(1 for t in path if (t.startswith("v_add_u32") or t.startswith("v_add3_u32")) and "%[c" in t)
+        assert n_acc == rows * 64 * 3 // 4 and n_ops >= n_acc

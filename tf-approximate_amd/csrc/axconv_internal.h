@@ -25,7 +25,7 @@ constexpr int kWaves = kBlockThreads / 64;
 // Accumulate instruction mix of the dense kernel's generated phase body (gen_lookup_asm.py emits the same):
 // 0 = one VALU add per table entry (v_add_u32 of a whole dword + v_add_u32_sdwa of its high half);
 // 1 = three per four entries (two dwords of one column pair folded by one v_add3_u32, the high halves by SDWA adds).
-constexpr int kDenseAccumulateMix = 0;
+constexpr int kDenseAccumulateMix = 1;   // what the 16- and 32-column tiles run (64-column tiles: mix 0)
 constexpr uint16_t kNullWeight = 256;          // slot that contributes nothing (padding channel / column)
 
 // Geometry of one dense layer after validation.

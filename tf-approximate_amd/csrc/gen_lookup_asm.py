@@ -102,19 +102,28 @@ def emit(nt, buf):
         off = " offset:128" if buf else ""
         return st.lds("ds_read_b128 v[%d:%d], v%d%s" % (b, b + 3, va, off))
 
-    def adds(st, r, step):
-        b = TEMP_BASE + 4 * step
-        g = step % sets
-        for e in range(8):
-            c = "%%[c%d_%d]" % (r, g * 8 + e)
-            if e % 2 == 0:
-                # the whole dword: the accumulator of the even column collects lo + 65536 * hi (mod 2^32); the
-                # kernel takes 65536 * (sum of hi) off again behind the last phase.  One plain add instead of an
-                # SDWA one.
-                st.ins("v_add_u32 %s, %s, v%d" % (c, c, b + e // 2))
+    def adds(st, r, steps):
+        """Accumulates the chunks of `steps` (one step, or two steps with the same column group)."""
+        g = steps[0] % sets
+        for d in range(4):
+            even = "%%[c%d_%d]" % (r, g * 8 + 2 * d)
+            odd = "%%[c%d_%d]" % (r, g * 8 + 2 * d + 1)
+            regs = [TEMP_BASE + 4 * step + d for step in steps]
+            # the whole dwords: the accumulator of the even column collects lo + 65536 * hi (mod 2^32); the kernel
+            # takes 65536 * (sum of hi) off again behind the last phase
+            if len(regs) == 2:
+                st.ins("v_add3_u32 %s, %s, v%d, v%d" % (even, even, regs[0], regs[1]))
             else:
+                st.ins("v_add_u32 %s, %s, v%d" % (even, even, regs[0]))
+            for reg in regs:
                 st.ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
-                       % (c, c, b + e // 2))
+                       % (odd, odd, reg))
+
+    # steps of a pixel that are accumulated together, in consumption order
+    if sets == 8:
+        groups = [(s,) for s in range(8)]
+    else:
+        groups = [(s, s + sets) for base in range(0, 8, 2 * sets) for s in range(base, base + sets)]
 
     def prime(st):
         src = rotate(st, 0)
@@ -123,14 +132,16 @@ def emit(nt, buf):
     def body(st, r, pending, with_next, state):
         """Accumulate pixel r (its reads are `pending`); with_next: refill the window with pixel r + 1.
         One auxiliary micro-operation is slotted in behind every chunk."""
-        nxt = []
+        nxt = [None] * 8
         src = rotate(st, r + 1) if with_next else None
-        for s in range(8):
-            st.wait(pending[s])
-            adds(st, r, s)
-            if with_next:
-                nxt.append(read(st, src, s))
-            aux_step(st, state)
+        for steps in groups:
+            # LDS operations complete in order: waiting for the youngest read of the group covers the others
+            st.wait(max((pending[s] for s in steps), key=lambda op: st.fifo.index(op) if op in st.fifo else -1))
+            adds(st, r, steps)
+            for s in steps:
+                if with_next:
+                    nxt[s] = read(st, src, s)
+                aux_step(st, state)
         return nxt
 
     # ---- auxiliary work, cut into micro-operations that are spread over the chunk slots ----
