@@ -320,6 +320,75 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
     psum[((int64_t)n * g.OH + oh) * g.OW + ow] = s;
 }
 
+// Patch sums for channel counts that are not a multiple of four (3-channel stems), same order and same results as
+// patch_sums_kernel.  A block owns `rb` consecutive output rows of one image: it copies the input rows under them
+// into LDS as they lie in memory (consecutive threads, consecutive floats), quantizes the rows it owns into the
+// code layout when xq is given (same ownership rule as patch_sums_rows_body), and then runs one sequential chain
+// per output pixel out of LDS, so every input float is fetched from memory about once instead of once per tap.
+__global__ void __launch_bounds__(1024) patch_sums_smallc_kernel(const float *__restrict__ x, const ConvGeom g,
+                                                                  const int rb, const int in_rows, const TensorQuant tq,
+                                                                  const LayerQuant *__restrict__ lq_dev,
+                                                                  float *__restrict__ psum, uint32_t *__restrict__ xq)
+{
+    const TensorQuant qt = lq_dev ? lq_dev->in : tq;
+    if (xq && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
+            xq[(int64_t)g.N * g.H * g.C4 * g.W + i] = qt.zp4;
+    extern __shared__ __align__(16) unsigned char ps_lds[];
+    float *const rows = reinterpret_cast<float *>(ps_lds);
+    const int t = threadIdx.x;
+    const int bands = (g.OH + rb - 1) / rb;
+    // consecutive bands (which share input rows) go to the same XCD: blocks are dealt round-robin over 8 XCDs
+    const int nblocks = (int)gridDim.x;
+    const int per_xcd = nblocks / 8, extra = nblocks % 8, xcd = (int)blockIdx.x & 7;
+    const int bid = xcd * per_xcd + (xcd < extra ? xcd : extra) + ((int)blockIdx.x >> 3);
+    const int n = bid / bands;
+    const int oh0 = (bid - n * bands) * rb;
+    const int ih_first = oh0 * g.sh - g.ph;  // input row held in LDS row 0 (may lie outside the image)
+    const int row_floats = g.W * g.C;
+    for (int i = t; i < in_rows * row_floats; i += blockDim.x) {
+        const int r = i / row_floats, e = i - r * row_floats;
+        const int ih = ih_first + r;
+        rows[i] = (unsigned)ih < (unsigned)g.H ? fake_quant_value(x[((int64_t)n * g.H + ih) * row_floats + e], qt) : 0.0f;
+    }
+    __syncthreads();
+    if (xq) {
+        const int own_lo = oh0 * g.sh;           // owned input rows: [own_lo, own_hi)
+        const int own_hi = (oh0 + rb >= g.OH) ? g.H : (oh0 + rb) * g.sh;
+        const int per_row = g.C4 * g.W;
+        for (int i = t; i < (own_hi - own_lo) * per_row; i += blockDim.x) {
+            const int ro = i / per_row, rem = i - ro * per_row;
+            const int c4 = rem / g.W, w = rem - c4 * g.W;
+            const int ih = own_lo + ro;
+            const float *src = &rows[(ih - ih_first) * row_floats + w * g.C + c4 * 4];
+            uint32_t packed = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (c4 * 4 + k < g.C)
+                    packed |= phys_row(quantize_code(src[k], qt.offset, qt.inv_scale)) << (8 * k);
+            xq[(((int64_t)n * g.H + ih) * g.C4 + c4) * g.W + w] = packed;
+        }
+    }
+    const int ohl = t / g.OW, ow = t - ohl * g.OW;
+    const int oh = oh0 + ohl;
+    if (ohl >= rb || oh >= g.OH)
+        return;
+    const int iw0 = ow * g.sw - g.pw;
+    float s = 0.0f;
+    for (int kh = 0; kh < g.KH; ++kh) {
+        const int r = ohl * g.sh + kh * g.dh;        // LDS row of this tap; rows outside the image hold zeros
+        for (int kw = 0; kw < g.KW; ++kw) {
+            const int iw = iw0 + kw * g.dw;
+            if ((unsigned)iw >= (unsigned)g.W)
+                continue;
+            const float *src = &rows[r * row_floats + iw * g.C];
+            for (int c = 0; c < g.C; ++c)
+                s = __fadd_rn(s, src[c]);
+        }
+    }
+    psum[((int64_t)n * g.OH + oh) * g.OW + ow] = s;
+}
+
 // Same relayout for caller-supplied codes (uint8 NHWC).
 __global__ void __launch_bounds__(256) codes_relayout_kernel(const uint8_t *__restrict__ codes, int64_t pixels,
                                                               int W, int C, int C4, uint32_t *__restrict__ xq)
@@ -1012,6 +1081,36 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 return e;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)), dim3(block_threads),
                                lds, stream, x, g, rb, in_rows, threads, tq, lq_dev, psum, fuse ? xq_fused : nullptr, fw);
+            return hipGetLastError();
+        }
+    }
+    if (!vec && g.OW <= 1024 && g.C < 64) {
+        // few channels that are not a multiple of four: bands of output rows with their input rows in LDS
+        const int64_t row_bytes = (int64_t)g.W * g.C * 4;
+        int rb = 0, in_rows = 0;
+        for (int cand = 1; cand <= g.OH && cand * g.OW <= 1024; ++cand) {
+            const int rows_needed = (cand - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+            if (rows_needed * row_bytes > 96 * 1024)
+                break;
+            if (cand > 1 && (int64_t)g.N * ((g.OH + cand - 1) / cand) < 1024)
+                break;
+            rb = cand;
+            in_rows = rows_needed;
+        }
+        if (rb > 0) {
+            int threads = ((rb * g.OW + 63) / 64) * 64;
+            threads = threads < 256 ? 256 : threads;
+            const bool fuse = xq_fused && fused && g.sh - 1 + g.ph <= (g.KH - 1) * g.dh &&
+                              (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1;
+            if (fuse)
+                *fused = true;
+            const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_smallc_kernel), 96 * 1024);
+            if (e != hipSuccess)
+                return e;
+            const int bands = (g.OH + rb - 1) / rb;
+            hipLaunchKernelGGL(patch_sums_smallc_kernel, dim3((unsigned)((int64_t)g.N * bands)), dim3(threads),
+                               (size_t)in_rows * row_bytes, stream, x, g, rb, in_rows, tq, lq_dev, psum,
+                               fuse ? xq_fused : nullptr);
             return hipGetLastError();
         }
     }
