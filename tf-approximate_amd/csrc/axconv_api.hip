@@ -629,6 +629,12 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     p.lq_dev = lq_dev;
     p.bias = bias;
     p.relu = activation == AXC_ACT_RELU ? 1 : 0;
+    {
+        const int64_t step = 64 * (kDenseWaves / 2), ohow = (int64_t)g.OH * g.OW;
+        p.step_n = (int)(step / ohow);
+        p.step_oh = (int)((step % ohow) / g.OW);
+        p.step_ow = (int)(step % g.OW);
+    }
     p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
     p.wq_bytes = (uint32_t)((size_t)pd.plan.n_col_tiles * pd.plan.fills * 128);
     if (pd.plan.k_splits > 1) {

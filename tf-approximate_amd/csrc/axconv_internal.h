@@ -95,6 +95,8 @@ struct DenseParams {
     float s1xs2, m1, m2, k_m1xm2; // epilogue constants; k_m1xm2 = float(K) * m1xM2
     uint32_t zp4;           // row-permuted zero code replicated in all four bytes
     uint32_t xq_bytes, wq_bytes; // sizes of the two streams (buffer-descriptor bounds)
+    int step_n, step_oh, step_ow; // 64 * kDenseWaves / 2 output pixels (the distance between a lane's pixels) as
+                                  // images, output rows and output columns
     const LayerQuant *lq_dev;    // not null: epilogue constants come from here instead of the four floats above
     const float *bias;           // not null: added to every output column after the epilogue
     int relu;                    // 1: max(x, 0) last

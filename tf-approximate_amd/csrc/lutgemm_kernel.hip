@@ -185,14 +185,13 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         if (rt != prev_rt) {
             prev_rt = rt;
             nr = 0;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int64_t wrow = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
-                nr += (wrow < row_end && wrow < wr_end) ? 1u : 0u;
-                const int64_t m = wrow + lane;
-                rvalid[r] = m < row_end && wrow < wr_end;
-                const int64_t mm = rvalid[r] ? m : row0;
-                int n, rem;
+            // (n, oh, ow) of this lane's first pixel by division; its further pixels lie a fixed number of output
+            // pixels apart (four wavefront-rows), so they follow by adding that step's (n, oh, ow) with carries
+            int n = 0, oh = 0, ow = 0;
+            {
+                const int64_t m0 = row0 + (int64_t)wr_base * 64 + lane;
+                const int64_t mm = m0 < g.M ? m0 : 0;
+                int rem;
                 if (g.M <= 0x7fffffff) { // the usual case: 32-bit divisions (a 64-bit one costs several times more)
                     const uint32_t ohow = (uint32_t)(g.OH * g.OW);
                     n = (int)((uint32_t)mm / ohow);
@@ -201,13 +200,28 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                     n = (int)(mm / ((int64_t)g.OH * g.OW));
                     rem = (int)(mm - (int64_t)n * g.OH * g.OW);
                 }
-                const int oh = (int)((uint32_t)rem / (uint32_t)g.OW);
-                const int ow = rem - oh * g.OW;
+                oh = (int)((uint32_t)rem / (uint32_t)g.OW);
+                ow = rem - oh * g.OW;
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int64_t wrow = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
+                nr += (wrow < row_end && wrow < wr_end) ? 1u : 0u;
+                const int64_t m = wrow + lane;
+                rvalid[r] = m < row_end && wrow < wr_end;
                 const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
                 // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
-                park[(2 * r) * kDenseThreads] = (uint32_t)((n * g.H + ih0) * rowstep + iw0);
+                park[(2 * r) * kDenseThreads] = rvalid[r] ? (uint32_t)((n * g.H + ih0) * rowstep + iw0) : 0u;
                 // input coordinates of tap (0, 0); ih0 = -32768 marks a pixel that does not exist
                 park[(2 * r + 1) * kDenseThreads] = rvalid[r] ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
+                // the next pixel of this lane: p.step_* = (n, oh, ow) of 64 * kDenseWaves / 2 output pixels
+                ow += p.step_ow;
+                const int c1 = ow >= g.OW ? 1 : 0;
+                ow -= c1 ? g.OW : 0;
+                oh += p.step_oh + c1;
+                const int c2 = oh >= g.OH ? 1 : 0;
+                oh -= c2 ? g.OH : 0;
+                n += p.step_n + c2;
             }
         }
 
