@@ -90,7 +90,8 @@ def _check_path(trace):
             lds.append(set(_regs(first)) if op.startswith("ds_read") else set())
             assert len(lds) <= 15, "more than 15 LDS operations in flight at %r" % text
         elif op.startswith("buffer_load"):
-            vm.append(set(_regs(TOKEN.search(text).group(0))))
+            # a load with the lds modifier lands in LDS, not in a register (its only register is the address)
+            vm.append(set() if text.rstrip().endswith(" lds") else set(_regs(TOKEN.search(text).group(0))))
     assert not lds and not vm, "operations still in flight at the end of the macro"
 
 

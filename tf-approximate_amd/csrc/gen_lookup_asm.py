@@ -16,12 +16,13 @@ barriers.  The macro interleaves, in one instruction stream with hand-counted s_
             source selector, the one in the low half by adding the whole dword (the surplus, 65536 times the
             high entries, is subtracted once behind the last phase).  Step s accumulates into column group
             s % (NT / 8).
-  stage     the table rows of fill p+2 (in ROWS since the previous phase) go to staged-row buffer BUF.
-  loads     table rows of fill p+3 -> ROWS (addresses from CODES), filter codes of fill p+4 -> CODES,
-            activations of fill p+1 -> ANEXT; waited for at the end of the macro.
+  loads     table rows of fill p+2 -> staged-row buffer BUF, straight from memory into LDS (buffer loads with the
+            lds modifier: M0 carries the LDS address of the wavefront's 1 KiB, every lane adds its 16 bytes;
+            addresses from CODES), filter codes of fill p+3 -> CODES, activations of fill p+1 -> ANEXT; all waited
+            for at the end of the macro.
   derive    the staged rows of fill p+1 (buffer BUF^1) are transposed into expanded-row buffer BUF^1: two
             items per lane, each four 8-byte reads, eight v_perm_b32 and four 8-byte writes.
-            Stage, loads and derive are cut into micro-operations and one of them is slotted in behind every
+            Loads and derive are cut into micro-operations and one of them is slotted in behind every
             16-byte chunk of the lookups (loads first, so that their latency runs under the lookups), so that
             the memory pipeline and the LDS see them spread out instead of as one burst per wavefront right
             after the barrier; what a wavefront with few pixels has not placed by its last chunk follows
@@ -145,19 +146,17 @@ def emit(nt, buf):
         return nxt
 
     # ---- auxiliary work, cut into micro-operations that are spread over the chunk slots ----
-    def stage_write(j):      # table rows of fill p+2: registers -> staged rows [buf]
-        return lambda st, state: st.lds("ds_write_b128 %%[sta], %%[w%d] offset:%d" % (j, j * 8192 + buf * 32768))
-
-    def row_load(j):         # table rows of fill p+3 <- table[code][16 bytes of this lane]
+    def row_load(j):         # staged rows [buf] of fill p+2 <- table[code][16 bytes of this lane], memory -> LDS
         def f(st, state):
             t = ADDR_BASE + 3    # the lookup address of a step is consumed by the read right behind it
+            st.ins("s_add_u32 m0, %%[stm], %d" % (j * 8192 + buf * 32768))
             st.ins("v_lshlrev_b32 v%d, 9, %%[k%d]" % (t, j))
             st.ins("v_and_or_b32 v%d, v%d, %%[cmask], %%[sto]" % (t, t))
-            st.ins("buffer_load_dwordx4 %%[w%d], v%d, %%[tab], 0 offen" % (j, t))
+            st.ins("buffer_load_dwordx4 v%d, %%[tab], 0 offen lds" % t)
             st.ins("s_nop 0")
         return f
 
-    def code_load(j):        # filter codes of fill p+4
+    def code_load(j):        # filter codes of fill p+3
         return lambda st, state: st.ins("buffer_load_ushort %%[k%d], %%[cvo], %%[wq], %%[cso] offen offset:%d" % (j, 32 * j))
 
     def act_load(r):         # activations of fill p+1
@@ -202,8 +201,8 @@ def emit(nt, buf):
     # a derive item five slots ahead of its transposes.
     aux = []
     for j in range(4):
-        aux += [both(stage_write(j), row_load(j))]      # row_load j reuses the registers stage_write j empties,
-    aux += [both(code_load(0), code_load(1)), both(code_load(2), code_load(3))]   # code_load j those of row_load j
+        aux += [row_load(j)]
+    aux += [both(code_load(0), code_load(1)), both(code_load(2), code_load(3))]   # code_load j overwrites what row_load j read
     aux += [both(act_load(r), act_load(r + 1)) for r in range(0, rows, 2)]
     aux += [derive_reads(0)]
     for _ in range(4):
@@ -252,14 +251,13 @@ def emit(nt, buf):
     zero.label("Lend_%=")
 
     outs = ['[c%d_%d] "+v"(ACC[%d][%d])' % (r, i, r, i) for r in range(rows) for i in range(nt)]
-    outs += ['[w%d] "+v"(ROWS[%d])' % (j, j) for j in range(4)]
     outs += ['[k%d] "+v"(CODES[%d])' % (j, j) for j in range(4)]
     outs += ['[n%d] "=&v"(ANEXT[%d])' % (r, r) for r in range(rows)]
     inp = ['[a%d] "v"(ACUR[%d])' % (r, r) for r in range(rows)]
     inp += ['[t%d] "v"(TAPOFF[%d])' % (r, r) for r in range(rows)]
     inp += ['[s%d] "v"(SEL[%d])' % (i, i) for i in range(8)]
     inp += ['[cha] "v"(CHA)', '[chb] "v"(CHB)', '[nr] "s"(NR)']
-    inp += ['[sta] "v"(STA)', '[sto] "v"(STO)', '[cvo] "v"(CVO)']
+    inp += ['[stm] "s"(STM)', '[sto] "v"(STO)', '[cvo] "v"(CVO)']
     inp += ['[rd0] "v"(RD[0])', '[rd1] "v"(RD[1])', '[wr0] "v"(WR[0])', '[wr1] "v"(WR[1])']
     inp += ['[plo] "s"(0x05040100u)', '[phi] "s"(0x07060302u)', '[cmask] "s"(0x01fffe00u)']
     inp += ['[tab] "s"(TAB)', '[wq] "s"(WQ)', '[xq] "s"(XQ)', '[cso] "s"(CSO)', '[qoff] "s"(QOFF)']
@@ -267,7 +265,7 @@ def emit(nt, buf):
         inp.append('[shift] "s"(SHIFT)')
     clob = ", ".join('"v%d"' % r for r in range(CLOBBER_FIRST, TEMP_BASE + 32))
     body_text = " \\\n        ".join(main.lines)
-    args = "ACC, ACUR, ANEXT, TAPOFF, ROWS, CODES, SEL, CHA, CHB, NR, SHIFT, STA, STO, CVO, RD, WR, TAB, WQ, XQ, CSO, QOFF"
+    args = "ACC, ACUR, ANEXT, TAPOFF, CODES, SEL, CHA, CHB, NR, SHIFT, STM, STO, CVO, RD, WR, TAB, WQ, XQ, CSO, QOFF"
     return ("#define PHASE_NT%d_B%d(%s) \\\n    asm volatile( \\\n        %s \\\n"
             "        : %s \\\n        : %s \\\n        : %s, \"scc\", \"memory\")\n"
             % (nt, buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))

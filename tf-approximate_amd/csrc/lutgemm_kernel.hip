@@ -13,8 +13,9 @@
 //   staged rows     2 x 32 KiB  the 64 table rows (512 contiguous bytes per filter code) of fill p + 1,
 //                               read bank-conflict free by the transposing lanes, while the rows of fill
 //                               p + 2 land in the other buffer
-// The table itself (128 KiB, resident in L2) is read with fully coalesced 16-byte loads, half a wavefront per
-// row, three fills ahead of the lookups; the filter codes that select the rows four fills ahead.
+// The table itself (128 KiB, resident in L2) is read with fully coalesced 16-byte loads that land in the staged
+// rows directly (buffer loads into LDS: no register, no LDS write instruction), half a wavefront per row, two
+// fills ahead of the lookups; the filter codes that select the rows three fills ahead.
 //
 // One workgroup of 8 wavefronts per CU, 256 VGPRs per wavefront: 128 int32 accumulators per lane
 // (R = 8 pixels x 16 columns, 4 x 32 or 2 x 64), eight 16-byte lookups in flight per wavefront.
@@ -63,31 +64,32 @@ struct DenseCfg {
 struct PhaseConsts {
     uint32_t sel[8];   // v_perm_b32 selectors that build the lookup address of step s
     uint32_t cha, chb; // packed chunk offsets of steps 0-3 / 4-7
-    uint32_t sta;      // LDS address of this thread's 16 bytes in staged row (thread / 32) of buffer 0
-    uint32_t sto;      // byte offset of those 16 bytes inside a 512-byte table row
+    uint32_t stm;      // LDS address of this wavefront's two staged rows (1 KiB) of buffer 0, load 0 (wave-uniform)
+    uint32_t sto;      // byte offset of this thread's 16 bytes inside a 512-byte table row
     uint32_t cvo;      // byte offset of filter code (thread / 32) inside the 64 codes of a fill
     uint32_t rd[2];    // LDS address (buffer 0) of the staged-row bytes derive item i reads
     uint32_t wr[2];    // LDS address (buffer 0) of the expanded-row bytes derive item i writes
 };
 
-// One phase (see gen_lookup_asm.py): lookups of fill p out of expanded-row buffer BUF, interleaved with staging
-// the rows of fill p+2, loading rows / codes / activations of later fills and expanding fill p+1.
+// One phase (see gen_lookup_asm.py): lookups of fill p out of expanded-row buffer BUF, interleaved with loading
+// the rows of fill p+2 into the staged rows, codes / activations of later fills, and expanding fill p+1.
 template <int NT, int BUF>
 __device__ __forceinline__ void phase_body(int32_t (&acc)[DenseCfg<NT>::R][NT], const uint32_t (&acur)[DenseCfg<NT>::R],
                                            uint32_t (&anext)[DenseCfg<NT>::R], const uint32_t (&tapoff)[DenseCfg<NT>::R],
-                                           u32x4 (&rows)[4], uint32_t (&codes)[4], const PhaseConsts &k,
+                                           uint32_t (&codes)[4], const PhaseConsts &k,
                                            const uint32_t nr, const uint32_t shift, const rsrc_t tab, const rsrc_t wq,
                                            const rsrc_t xq, const uint32_t cso, const uint32_t qoff)
 {
+    const uint32_t stm = __builtin_amdgcn_readfirstlane(k.stm);
     if constexpr (NT == 16) {
-        if constexpr (BUF == 0) PHASE_NT16_B0(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
-        else PHASE_NT16_B1(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        if constexpr (BUF == 0) PHASE_NT16_B0(acc, acur, anext, tapoff, codes, k.sel, k.cha, k.chb, nr, shift, stm, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        else PHASE_NT16_B1(acc, acur, anext, tapoff, codes, k.sel, k.cha, k.chb, nr, shift, stm, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
     } else if constexpr (NT == 32) {
-        if constexpr (BUF == 0) PHASE_NT32_B0(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
-        else PHASE_NT32_B1(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        if constexpr (BUF == 0) PHASE_NT32_B0(acc, acur, anext, tapoff, codes, k.sel, k.cha, k.chb, nr, shift, stm, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        else PHASE_NT32_B1(acc, acur, anext, tapoff, codes, k.sel, k.cha, k.chb, nr, shift, stm, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
     } else {
-        if constexpr (BUF == 0) PHASE_NT64_B0(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
-        else PHASE_NT64_B1(acc, acur, anext, tapoff, rows, codes, k.sel, k.cha, k.chb, nr, shift, k.sta, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        if constexpr (BUF == 0) PHASE_NT64_B0(acc, acur, anext, tapoff, codes, k.sel, k.cha, k.chb, nr, shift, stm, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
+        else PHASE_NT64_B1(acc, acur, anext, tapoff, codes, k.sel, k.cha, k.chb, nr, shift, stm, k.sto, k.cvo, k.rd, k.wr, tab, wq, xq, cso, qoff);
     }
 }
 
@@ -272,15 +274,15 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 codes[j] = __builtin_amdgcn_raw_buffer_load_b16(wq_rsrc, (int)((st_slot + 16u * j) * 2u),
                                                                 (int)(wq_tile + f * 128u), 0);
         };
-        auto load_rows = [&](const uint32_t (&codes)[4], u32x4 (&rows)[4]) {
+        // table rows of one fill -> staged rows [buf], straight from memory into LDS: the wavefront's 64 lanes
+        // fill 1 KiB (two rows) per load, lane l the 16 bytes at l * 16
+        auto load_rows_to_stage = [&](const uint32_t (&codes)[4], const uint32_t buf) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                rows[j] = __builtin_amdgcn_raw_buffer_load_b128(tab_rsrc, (int)((codes[j] & 0xffffu) * 512u + st_off), 0, 0);
-        };
-        auto store_stage = [&](const u32x4 (&rows)[4], const uint32_t buf) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                *reinterpret_cast<u32x4 *>(stage + buf * kExpandBytes + (st_slot + 16u * j) * 512u + st_off) = rows[j];
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    tab_rsrc,
+                    (__attribute__((address_space(3))) void *)(stage + buf * kExpandBytes + 16u * j * 512u + (uint32_t)wave * 1024u),
+                    16, (int)((codes[j] & 0xffffu) * 512u + st_off), 0, 0, 0);
         };
         auto derive = [&](const uint32_t buf) { // staged rows [buf] -> expanded rows [buf]
 #pragma unroll
@@ -306,28 +308,22 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
 
         // ---- prologue ----
         // state entering phase p: expanded rows of fill p in D[p & 1]; staged rows of fill p+1 in S[(p+1) & 1];
-        // rows = table rows of fill p+2 (in flight); codes = filter codes of fill p+3 (in flight);
-        // acts[p & 1] = activations of fill p
+        // codes = filter codes of fill p+2 (in flight); acts[p & 1] = activations of fill p
         uint32_t actA[R], actB[R];
-        u32x4 rows[4];
         uint32_t codes[4];
         tap_setup();
         load_acts(actA);
         {
-            // two rounds of loads, each in flight together: the filter codes of fills 0-3, then the table rows
-            // of fills 0-2 (the accumulators are not live yet, so the registers are there)
-            uint32_t codes0[4], codes1[4], codes2[4];
-            u32x4 rows0[4], rows1[4];
+            // two rounds of loads, each in flight together: the filter codes of fills 0-2, then the table rows
+            // of fills 0 and 1, which go straight into the two staged-row buffers
+            uint32_t codes0[4], codes1[4];
             load_codes(0, codes0);
             load_codes(1, codes1);
-            load_codes(2, codes2);
-            load_codes(3, codes);
-            load_rows(codes0, rows0);
-            load_rows(codes1, rows1);
-            load_rows(codes2, rows);
+            load_codes(2, codes);
             __syncthreads();          // the previous tile's last phase and epilogue are done with every buffer
-            store_stage(rows0, 0);
-            store_stage(rows1, 1);
+            load_rows_to_stage(codes0, 0);
+            load_rows_to_stage(codes1, 1);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         __syncthreads();
         derive(0);
@@ -347,7 +343,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             k.sel[i] = sel[i];
         k.cha = cha;
         k.chb = chb;
-        k.sta = 2u * kExpandBytes + st_slot * 512u + st_off;
+        k.stm = 2u * kExpandBytes + (uint32_t)wave * 1024u;
         k.sto = st_off;
         k.cvo = st_slot * 2u;
 #pragma unroll
@@ -363,10 +359,10 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             advance_cursor();
         auto phase = [&](const int pcur, uint32_t (&act_cur)[R], uint32_t (&act_next)[R], auto buf_tag) {
             constexpr int BUF = decltype(buf_tag)::value;
-            const int fcodes = pcur + 4 < fills_left ? pcur + 4 : fills_left - 1;
+            const int fcodes = pcur + 3 < fills_left ? pcur + 3 : fills_left - 1;
             const uint32_t cso = wq_tile + (uint32_t)fcodes * 128u;
             const uint32_t qoff = (uint32_t)(cur_q * g.W * 4);
-            phase_body<NT, BUF>(acc, act_cur, act_next, idx_tap, rows, codes, k, nr_s,
+            phase_body<NT, BUF>(acc, act_cur, act_next, idx_tap, codes, k, nr_s,
                                 __builtin_amdgcn_readfirstlane(shift_cur), tab_rsrc, wq_rsrc, xq_rsrc,
                                 __builtin_amdgcn_readfirstlane(cso), __builtin_amdgcn_readfirstlane(qoff));
             shift_cur = (uint32_t)cur_sub * (32u / SUBS); // bits to rotate the channels of fill pcur+1 down
