@@ -198,17 +198,17 @@ def emit(nt, buf):
 
     # Global loads first: a wavefront with few pixels has few chunk slots, and what does not fit behind a chunk is
     # issued behind the last one, right in front of the wait for it.  Then the expansion of fill p+1, the reads of
-    # a derive item five slots ahead of its transposes.
+    # a derive item eight slots ahead of its transposes.
     aux = []
     for j in range(4):
         aux += [row_load(j)]
     aux += [both(code_load(0), code_load(1)), both(code_load(2), code_load(3))]   # code_load j overwrites what row_load j read
     aux += [both(act_load(r), act_load(r + 1)) for r in range(0, rows, 2)]
     aux += [derive_reads(0)]
-    for _ in range(4):
+    for _ in range(7):
         aux.append(lambda st, state: None)
     aux += [both(derive_consume(0), derive_reads(1))]
-    for _ in range(4):
+    for _ in range(7):
         aux.append(lambda st, state: None)
     aux += [derive_consume(1)]
 
