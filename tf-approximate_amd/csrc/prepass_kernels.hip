@@ -3,6 +3,24 @@
 
 namespace axc {
 
+// Keeps the LDS reads and the adds (into `sum`) around it in program order, in the compiler's own passes and in its
+// scheduler: the empty statement claims to read and write both memory and the running sum.
+__device__ __forceinline__ void chain_fence(float &sum)
+{
+    __asm__ volatile("" : "+v"(sum) : : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Waits until at most `pending` LDS reads of this wavefront are outstanding (they return in order).  A lone wavefront
+// issues about one instruction per four cycles whatever its kind, so one wait per batch of reads instead of one per
+// read is time the chain gets back.
+template <int PENDING>
+__device__ __forceinline__ void wait_lds_reads()
+{
+    static_assert(PENDING >= 0 && PENDING <= 15, "lgkmcnt is a 4-bit counter");
+    __builtin_amdgcn_s_waitcnt(0xC07F | (PENDING << 8)); // vmcnt and expcnt left at their maxima
+}
+
 // Input pre-pass.  Restates the quantize and the channel part of the patch sum of
 // ApproxConvIm2ColKernel (tf2/src/approx_nn_conv_kernels.cpp:288-294) once per input element
 // instead of once per patch element.
@@ -210,6 +228,29 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
         psum[m] = s;
 }
 
+// The filter pre-pass of a layer is independent of its input pre-pass: as two launches they would run one after
+// the other, so the launch below carries both.  The first filter_blocks8 workgroups (a multiple of 8, which keeps
+// workgroup index mod 8 = XCD for the others) do the filter work of filter_prep_kernel, the rest the patch sums.
+struct FilterWork {
+    const float *filter;
+    const uint8_t *filter_codes;
+    int taps, C, C4, Co, nt, n_col_tiles;
+    TensorQuant tq;
+    uint16_t *wq;
+    int sum_blocks;
+    float *fsum;
+    int blocks;    // sum_blocks + pack blocks; 0: no filter work in this launch
+    int blocks8;   // blocks rounded up to a multiple of 8
+    // pack_total > 0: no pack blocks; the threads of the patch-sum blocks that run no chain pack the codes,
+    // each block its share of the pack_total elements
+    int64_t pack_total;
+};
+
+__device__ __forceinline__ void filter_pack_element(const int64_t i, const float *__restrict__ filter,
+                                                    const uint8_t *__restrict__ filter_codes, int taps, int C,
+                                                    int C4, int Co, int nt, int n_col_tiles, const TensorQuant &qf,
+                                                    uint16_t *__restrict__ wq);
+
 // Patch sums for C % 4 == 0 when the input rows under a band of output rows fit in LDS: same order and same
 // results as patch_sums_kernel.  A block owns `rb` consecutive output rows of one image (one thread per output
 // pixel) and first copies the input rows they touch into LDS, so every input float is fetched from memory
@@ -221,7 +262,7 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
                                                      const int in_rows, const TensorQuant &tq,
                                                      const LayerQuant *__restrict__ lq_dev, float *__restrict__ psum,
                                                      uint32_t *__restrict__ xq, const int bid_in, const int nblocks,
-                                                     const int nthreads)
+                                                     const int nthreads, const FilterWork &fw)
 {
     // xq != nullptr: the block also quantizes the input rows it owns among those it copies (the rows under its
     // own band of output rows; the launcher has checked that these lie inside every block's window and together
@@ -246,37 +287,47 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
     if (t >= nthreads) {
         // not taking part in the copy
     } else if (nthreads % g.C4 == 0) {
-        // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns, four
-        // 16-byte loads in flight at a time
+        // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns, sixteen
+        // 16-byte loads in flight at a time.  The loads are unconditional (coordinates clamped into the image, the
+        // result replaced by zeros afterwards) so that each store waits for its own load only.
+        constexpr int kInFlight = 16;
         const int q = t % g.C4, w0 = t / g.C4, wstep = nthreads / g.C4;
         const int wsteps = (g.W + wstep - 1) / wstep;
         const int iters = in_rows * wsteps;
-        for (int it0 = 0; it0 < iters; it0 += 4) {
-            float4 v[4];
-            int rr[4], ww[4];
+        const float *const xn = x + (int64_t)n * g.H * g.W * g.C + q * 4;
+        int r_next = 0, ws_next = 0; // (row, column step) of the next item
+        for (int it0 = 0; it0 < iters; it0 += kInFlight) {
+            float4 v[kInFlight];
+            int rr[kInFlight], ww[kInFlight];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int it = it0 + u;
-                rr[u] = it / wsteps;
-                ww[u] = w0 + (it - rr[u] * wsteps) * wstep;
-                const int ih = ih_first + rr[u];
-                v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                if (it < iters && ww[u] < g.W && (unsigned)ih < (unsigned)g.H)
-                    v[u] = *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + ww[u]) * g.C + q * 4);
+            for (int u = 0; u < kInFlight; ++u) {
+                rr[u] = r_next;
+                ww[u] = w0 + ws_next * wstep;
+                if (++ws_next == wsteps) {
+                    ws_next = 0;
+                    ++r_next;
+                }
+                int ih = ih_first + rr[u];
+                ih = ih < 0 ? 0 : (ih >= g.H ? g.H - 1 : ih);
+                const int wc = ww[u] < g.W ? ww[u] : g.W - 1;
+                v[u] = *reinterpret_cast<const float4 *>(xn + ((int64_t)ih * g.W + wc) * g.C);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (it0 + u >= iters || ww[u] >= g.W)
-                    continue;
+            for (int u = 0; u < kInFlight; ++u) {
                 const int ih = ih_first + rr[u];
-                const float4 f = fake_quant_value4(v[u], qt);   // rows outside the image stay zero
-                *reinterpret_cast<float4 *>(&rows[(rr[u] * g.W + ww[u]) * pitch + q * 4]) = f;
-                if (xq && (unsigned)ih < (unsigned)g.H && ih >= own_lo && ih < own_hi)
-                    xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + ww[u]] =
-                        phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
-                        (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
-                        (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
-                        (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
+                const bool in_image = (unsigned)ih < (unsigned)g.H;
+                float4 f = fake_quant_value4(v[u], qt);
+                if (!in_image)
+                    f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);   // rows outside the image are zeros
+                if (it0 + u < iters && ww[u] < g.W) {
+                    *reinterpret_cast<float4 *>(&rows[(rr[u] * g.W + ww[u]) * pitch + q * 4]) = f;
+                    if (xq && in_image && ih >= own_lo && ih < own_hi)
+                        xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + ww[u]] =
+                            phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
+                            (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
+                            (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
+                            (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
+                }
             }
         }
     } else {
@@ -293,13 +344,97 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
             *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
         }
     }
+    float *const zero_px = rows + (size_t)in_rows * g.W * pitch; // one pixel of zeros behind the rows (see below)
+    if (t < g.C4)
+        *reinterpret_cast<float4 *>(zero_px + t * 4) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     __syncthreads();
-    const int ohl = t / g.OW, ow = t - ohl * g.OW;
+    // Chains go to the wavefronts of the block starting from a different one in blocks that are likely to share a
+    // CU (wavefronts of a block are spread over the SIMDs in order), so that their chains do not share a SIMD.
+    const int rot = ((bid_in >> 8) + (bid_in >> 3)) & 3;
+    const int tc = (t + (int)blockDim.x - rot * 64) % (int)blockDim.x;
+    const int ohl = tc / g.OW, ow = tc - ohl * g.OW;
     const int oh = oh0 + ohl;
-    if (ohl >= rb || oh >= g.OH)
+    if (ohl >= rb) {
+        // No chain for this thread.  If the launch asks for it, it packs filter codes meanwhile - but only from
+        // wavefronts that share no SIMD with a chain (wavefront w of the block sits on SIMD w mod 4): a chain
+        // runs as fast as its wavefront gets to issue, and any other work on its SIMD takes issue slots from it.
+        const int chain_waves = (rb * g.OW + 63) / 64;
+        const int wave = tc >> 6; // counted from the first chain wavefront
+        if (fw.pack_total > 0 && (wave & 3) >= chain_waves) {
+            const int waves = (int)blockDim.x >> 6;
+            const int free_simds = 4 - chain_waves; // the launcher asks for this work only when chain_waves < 4
+            const int workers = ((waves >> 2) * free_simds) * 64; // blockDim.x is 512 or 1024: 2 or 4 wavefronts per SIMD
+            const int widx = (((wave >> 2) * free_simds + (wave & 3) - chain_waves) << 6) + (tc & 63);
+            const int64_t share = (((fw.pack_total + nblocks - 1) / nblocks) + 63) & ~(int64_t)63;
+            const int64_t first = (int64_t)bid_in * share;
+            const int64_t last = first + share < fw.pack_total ? first + share : fw.pack_total;
+            const TensorQuant qf = lq_dev ? lq_dev->flt : fw.tq;
+            for (int64_t i = first + widx; i < last; i += workers)
+                filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt,
+                                    fw.n_col_tiles, qf, fw.wq);
+        }
+        return;
+    }
+    if (oh >= g.OH)
         return;
     const int iw0 = ow * g.sw - g.pw;
     float s = 0.0f;
+    if ((g.C4 & 7) == 0) {
+        // The chain of K dependent adds is what takes the time here, so nothing else may wait on it: the taps and
+        // their channels form one flat list of batches of 32 floats, the LDS reads of a batch are issued a batch
+        // ahead of its adds, and every lane takes every tap - a tap outside the image reads the pixel of zeros
+        // (x + 0 == x; the sum starts at +0 and so is never -0) instead of branching around it.
+        constexpr int kBatch = 8; // 16-byte reads per batch
+        const int bpt = g.C4 / kBatch, nb = g.KH * g.KW * bpt;
+        int kh = 0, kw = 0, bi = 0;
+        auto tap_src = [&]() -> const float4 * {
+            const int iw = iw0 + kw * g.dw;
+            const bool ok = kh < g.KH && (unsigned)iw < (unsigned)g.W;
+            return reinterpret_cast<const float4 *>(ok ? rows + ((ohl * g.sh + kh * g.dh) * g.W + iw) * pitch : zero_px);
+        };
+        const float4 *src = tap_src();
+        auto read = [&](float4(&w)[kBatch]) {
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i)
+                w[i] = src[bi * kBatch + i];
+            if (++bi == bpt) { // next tap (beyond the last one: the pixel of zeros, read but never added)
+                bi = 0;
+                if (++kw == g.KW) {
+                    kw = 0;
+                    ++kh;
+                }
+                src = tap_src();
+            }
+        };
+        auto add = [&](const float4(&w)[kBatch]) {
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                s = __fadd_rn(s, w[i].x);
+                s = __fadd_rn(s, w[i].y);
+                s = __fadd_rn(s, w[i].z);
+                s = __fadd_rn(s, w[i].w);
+            }
+        };
+        float4 w0[kBatch], w1[kBatch];
+        read(w0);
+        for (int b = 0; b < nb; b += 2) {
+            // the scheduling fences keep each read behind the adds that free its registers: hoisted above them it
+            // would need a third register set and a copy back at the end of every iteration
+            read(w1);
+            chain_fence(s);
+            wait_lds_reads<kBatch>();
+            add(w0);
+            chain_fence(s);
+            read(w0);
+            chain_fence(s);
+            wait_lds_reads<kBatch>();
+            if (b + 1 < nb)
+                add(w1);
+            chain_fence(s);
+        }
+        psum[((int64_t)n * g.OH + oh) * g.OW + ow] = s;
+        return;
+    }
     for (int kh = 0; kh < g.KH; ++kh) {
         const int r = ohl * g.sh + kh * g.dh;        // LDS row of this tap; rows outside the image hold zeros,
         for (int kw = 0; kw < g.KW; ++kw) {          // and x + 0.0f == x, so they need no branch
@@ -445,13 +580,17 @@ __device__ __forceinline__ void filter_pack_element(const int64_t i, const float
     wq[i] = code;
 }
 
-// Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one thread per output column,
-// rows (h, w, c) ascending.
-// A block owns 64 columns; all its threads (512 or 1024) stage up to 256 filter rows at a time into LDS (coalesced, every
-// load of a pass in flight at once), then the first 64 threads extend their column's sequential sum from LDS,
-// 32 independent LDS reads ahead of the dependent chain of adds.
-constexpr int kFsRows = 256, kFsThreads = 1024; // 65 KiB of LDS: a launch that also does patch sums keeps their LDS size
-constexpr int kFsLdsBytes = kFsRows * 65 * 4;
+// Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one sequential sum per output column, rows (h, w, c)
+// ascending.  The chain of K dependent adds sets the time, so everything else is kept off it, and memory latency
+// is covered by volume in flight: a block owns only kFsCols columns (64-byte pieces of filter rows), which leaves
+// each of its loads a whole row of lead.  It walks the filter rows in passes of kFsRows: all its threads (512 or
+// 1024) load a pass kFsAhead passes ahead of its use and store it into one half of an LDS stage; meanwhile the
+// first kFsCols lanes extend the sums from the other half.  A lone wavefront issues about one instruction every
+// four cycles whatever its kind, so the stage is column-major and a lane fetches four rows per LDS read, one batch
+// of 16 rows ahead of the adds: 21 instructions per 16 adds.  One barrier per pass.  Rows beyond K are staged as zeros and summed like the others: the sums start at +0 and
+// so are never -0, and x + 0 == x.
+constexpr int kFsCols = 16, kFsRows = 256, kFsPitch = kFsRows + 4, kFsAhead = 3, kFsThreads = 1024;
+constexpr int kFsLdsBytes = 2 * kFsCols * kFsPitch * 4; // 32.5 KiB: two halves of [column][row], rows padded by 4
 
 extern __shared__ __align__(16) unsigned char fs_lds[];
 
@@ -459,46 +598,91 @@ template <int THREADS>
 __device__ __forceinline__ void filter_sums_block(const int block, const float *__restrict__ filter, int K, int Co,
                                                   const TensorQuant &q, float *__restrict__ fsum)
 {
-    constexpr int kBatch = 32, kPer = kFsRows * 64 / THREADS; // loads per thread per pass
+    constexpr int kBatch = 16, kStep = THREADS / kFsCols, kPer = kFsRows / kStep; // loads per thread per pass
     float *const stage = reinterpret_cast<float *>(fs_lds);
-    const int col0 = block * 64;
+    const int col0 = block * kFsCols;
     const int t = threadIdx.x;
-    const int cl = t & 63, rsub = t >> 6; // THREADS / 64 rows per step
-    float s = 0.0f;
-    for (int k0 = 0; k0 < K; k0 += kFsRows) {
-        float v[kPer];
+    const int cl = t % kFsCols, rsub = t / kFsCols;
+    const bool col_ok = col0 + cl < Co;
+    const float *const src = filter + (col_ok ? col0 + cl : Co - 1);
+    const int npass = (K + kFsRows - 1) / kFsRows;
+    // Loads and stores below are unconditional (rows beyond K load row K - 1 and are stored as zeros, passes beyond
+    // the last likewise), so that the loop body is straight-line code for the compiler's count of loads in flight:
+    // a store then waits for its own pass only, not for the passes issued after it.
+    float v[kFsAhead][kPer];
+    auto issue = [&](float(&dst)[kPer], int pass) {
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
-            const int k = k0 + rsub + i * (THREADS / 64);
-            v[i] = (k < K && col0 + cl < Co) ? filter[(int64_t)k * Co + col0 + cl] : 0.0f;
+            const int k = pass * kFsRows + rsub + i * kStep;
+            dst[i] = src[(int64_t)(k < K ? k : K - 1) * Co];
         }
-        if (q.fq) { // after the loads, so that they all stay in flight together
+    };
+    auto store = [&](const float(&from)[kPer], int pass) {
+        float *const half = stage + (pass & 1) * (kFsCols * kFsPitch);
 #pragma unroll
-            for (int i = 0; i < kPer; ++i)
-                v[i] = fake_quant_value(v[i], q);   // padding zeros lie on the grid or are never summed
+        for (int i = 0; i < kPer; ++i) {
+            const int r = rsub + i * kStep;
+            float f = from[i];
+            if (q.fq)
+                f = fake_quant_value(f, q);
+            half[cl * kFsPitch + r] = (pass * kFsRows + r < K) ? f : 0.0f;
         }
-        __syncthreads(); // previous pass consumed
+    };
 #pragma unroll
-        for (int i = 0; i < kPer; ++i)
-            stage[(rsub + i * (THREADS / 64)) * 65 + cl] = v[i];
-        __syncthreads();
-        if (t < 64) {
-            const int nr = (K - k0 < kFsRows) ? K - k0 : kFsRows;
-            int r = 0;
-            for (; r + kBatch <= nr; r += kBatch) {
-                float w[kBatch];
+    for (int u = 0; u < kFsAhead; ++u)
+        issue(v[u], u);
+    store(v[0], 0);
+    issue(v[0], kFsAhead);
+    __syncthreads();
+    float s = 0.0f;
+    // one pass: `next` holds pass p + 1 (stored now, then refilled with the loads of pass p + 1 + kFsAhead);
+    // pass p lies in its half of the stage
+    auto pass_step = [&](const int p, float(&next)[kPer]) {
+        store(next, p + 1);
+        issue(next, p + 1 + kFsAhead);
+        if (t < kFsCols && p < npass) {
+            const float4 *const half = reinterpret_cast<const float4 *>(stage + (p & 1) * (kFsCols * kFsPitch) + t * kFsPitch);
+            const int left = K - p * kFsRows;
+            const int nb = left >= kFsRows ? kFsRows / kBatch : (left + kBatch - 1) / kBatch;
+            float4 w0[kBatch / 4], w1[kBatch / 4];
+            auto read = [&](float4(&w)[kBatch / 4], int b) {
 #pragma unroll
-                for (int i = 0; i < kBatch; ++i)
-                    w[i] = stage[(r + i) * 65 + t];
+                for (int i = 0; i < kBatch / 4; ++i)
+                    w[i] = half[b * (kBatch / 4) + i];
+            };
+            auto add = [&](const float4(&w)[kBatch / 4]) {
 #pragma unroll
-                for (int i = 0; i < kBatch; ++i)
-                    s = __fadd_rn(s, w[i]);
+                for (int i = 0; i < kBatch / 4; ++i) {
+                    s = __fadd_rn(s, w[i].x);
+                    s = __fadd_rn(s, w[i].y);
+                    s = __fadd_rn(s, w[i].z);
+                    s = __fadd_rn(s, w[i].w);
+                }
+            };
+            read(w0, 0);
+            for (int b = 0; b < nb; b += 2) { // nb is even or 1; reads beyond the pass's rows stay inside the stage
+                read(w1, b + 1);
+                chain_fence(s);
+                wait_lds_reads<kBatch / 4>();
+                add(w0);
+                chain_fence(s);
+                read(w0, b + 2 < kFsRows / kBatch ? b + 2 : 0);
+                chain_fence(s);
+                wait_lds_reads<kBatch / 4>();
+                if (b + 1 < nb)
+                    add(w1);
+                chain_fence(s);
             }
-            for (; r < nr; ++r)
-                s = __fadd_rn(s, stage[r * 65 + t]);
         }
+        __syncthreads();
+    };
+    static_assert(kFsAhead == 3, "the pass loop below rotates three register sets");
+    for (int p0 = 0; p0 < npass; p0 += kFsAhead) {
+        pass_step(p0, v[1]);
+        pass_step(p0 + 1, v[2]);
+        pass_step(p0 + 2, v[0]);
     }
-    if (t < 64 && col0 + t < Co)
+    if (t < kFsCols && col_ok)
         fsum[col0 + t] = s;
 }
 
@@ -612,20 +796,140 @@ __device__ __forceinline__ void patch_sums_flat_body(const float *__restrict__ x
         psum[m0 + t] = s;
 }
 
-// The filter pre-pass of a layer is independent of its input pre-pass: as two launches they would run one after
-// the other, so the launch below carries both.  The first filter_blocks8 workgroups (a multiple of 8, which keeps
-// workgroup index mod 8 = XCD for the others) do the filter work of filter_prep_kernel, the rest the patch sums.
-struct FilterWork {
-    const float *filter;
-    const uint8_t *filter_codes;
-    int taps, C, C4, Co, nt, n_col_tiles;
-    TensorQuant tq;
-    uint16_t *wq;
-    int sum_blocks;
-    float *fsum;
-    int blocks;    // sum_blocks + pack blocks; 0: no filter work in this launch
-    int blocks8;   // blocks rounded up to a multiple of 8
-};
+// The flat pixel list with many channels and few pixels (the deep, small layers of a network): there the chain of
+// C dependent adds per pixel is what takes the time, and memory latency has to stay off it.  A workgroup takes
+// `pixels` (8 or 16) consecutive pixels, so that even a few thousand pixels spread over all CUs, and walks their
+// channels in passes of kDeepChunk: all threads load a pass kDeepAhead passes ahead of its use (16 bytes per lane,
+// a wavefront fetches 1 KiB of one pixel), quantize it into the code layout when xq is given and store it into
+// one half of an LDS stage [pixel][channel]; meanwhile one lane per pixel extends its sum from the other half,
+// its 16-byte LDS reads a batch of 32 channels ahead of the adds.  One barrier per pass.  Loads, stores and LDS
+// reads are unconditional (indices clamped, zeros stored beyond C) to keep the loop body straight-line code for
+// the compiler's count of loads in flight: a store then waits for its own pass only.
+constexpr int kDeepChunk = 256, kDeepPitch = kDeepChunk + 4, kDeepAhead = 3, kDeepThreads = 512;
+constexpr int deep_lds_bytes(int pixels) { return 2 * pixels * kDeepPitch * 4; }
+
+template <int PIXELS>
+__device__ __forceinline__ void patch_sums_deep_body(const float *__restrict__ x, const ConvGeom &g,
+                                                     const TensorQuant &tq, const LayerQuant *__restrict__ lq_dev,
+                                                     float *__restrict__ psum, uint32_t *__restrict__ xq,
+                                                     const int bid)
+{
+    constexpr int pixels = PIXELS, kDeepMaxPixels = PIXELS;
+    constexpr int kDeepPer = PIXELS * (kDeepChunk / 4) / kDeepThreads; // 16-byte loads per thread and pass
+    const TensorQuant qt = lq_dev ? lq_dev->in : tq;
+    if (xq && bid == 0)
+        for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
+            xq[(int64_t)g.N * g.H * g.C4 * g.W + i] = qt.zp4;
+    extern __shared__ __align__(16) unsigned char pd_lds[];
+    float *const stage = reinterpret_cast<float *>(pd_lds);
+    const int t = threadIdx.x;
+    const int64_t m0 = (int64_t)bid * pixels;
+    const int npx = (int)(g.M - m0 < pixels ? g.M - m0 : pixels);
+    constexpr int QUADS = kDeepChunk / 4, PSTEP = kDeepThreads / QUADS;
+    const int q = t % QUADS, px0 = t / QUADS;
+    const bool loader = t < kDeepThreads;
+    const int npass = (g.C + kDeepChunk - 1) / kDeepChunk;
+    const float *src[kDeepPer];
+    uint32_t xq_idx[kDeepPer];
+    bool px_ok[kDeepPer];
+#pragma unroll
+    for (int k = 0; k < kDeepPer; ++k) {
+        const int px = px0 + k * PSTEP;
+        px_ok[k] = loader && px < npx;
+        const int64_t m = m0 + (px < npx ? px : npx - 1);
+        const int64_t nh = m / g.W;
+        const int w = (int)(m - nh * g.W);
+        xq_idx[k] = (uint32_t)((nh * g.C4 + q) * g.W + w);
+        src[k] = x + m * g.C;
+    }
+    float4 v[kDeepAhead][kDeepPer];
+    auto issue = [&](float4(&dst)[kDeepPer], int pass) {
+        const int c = pass * kDeepChunk + q * 4;
+        const int cc = c < g.C ? c : g.C - 4;
+#pragma unroll
+        for (int k = 0; k < kDeepPer; ++k)
+            dst[k] = *reinterpret_cast<const float4 *>(src[k] + cc);
+    };
+    auto store = [&](const float4(&from)[kDeepPer], int pass) {
+        float *const half = stage + (pass & 1) * (kDeepMaxPixels * kDeepPitch);
+        const bool c_ok = pass * kDeepChunk + q * 4 < g.C;
+#pragma unroll
+        for (int k = 0; k < kDeepPer; ++k) {
+            const int px = px0 + k * PSTEP;
+            float4 f = fake_quant_value4(from[k], qt);
+            if (!c_ok)
+                f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (loader && px < kDeepMaxPixels)
+                *reinterpret_cast<float4 *>(&half[px * kDeepPitch + q * 4]) = f;
+            if (xq && px_ok[k] && c_ok)
+                xq[xq_idx[k] + (uint32_t)(pass * (kDeepChunk / 4)) * (uint32_t)g.W] =
+                    phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
+                    (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
+                    (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
+                    (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < kDeepAhead; ++u)
+        issue(v[u], u);
+    store(v[0], 0);
+    if (kDeepAhead < npass)
+        issue(v[0], kDeepAhead);
+    __syncthreads();
+    float s = 0.0f;
+    constexpr int kBatch = 8, kBatches = QUADS / kBatch; // 16-byte reads per batch; batches per pass
+    auto pass_step = [&](const int p, float4(&next)[kDeepPer]) {
+        store(next, p + 1);
+        if (p + 1 + kDeepAhead < npass)
+            issue(next, p + 1 + kDeepAhead);
+        if (t < kDeepMaxPixels && p < npass) {
+            const float4 *const row =
+                reinterpret_cast<const float4 *>(stage + (p & 1) * (kDeepMaxPixels * kDeepPitch) + t * kDeepPitch);
+            float4 w0[kBatch], w1[kBatch];
+            auto read = [&](float4(&w)[kBatch], int b) {
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i)
+                    w[i] = row[b * kBatch + i];
+            };
+            auto add = [&](const float4(&w)[kBatch]) {
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i) {
+                    s = __fadd_rn(s, w[i].x);
+                    s = __fadd_rn(s, w[i].y);
+                    s = __fadd_rn(s, w[i].z);
+                    s = __fadd_rn(s, w[i].w);
+                }
+            };
+            read(w0, 0);
+#pragma unroll
+            for (int b = 0; b < kBatches; b += 2) {
+                read(w1, b + 1);
+                chain_fence(s);
+                wait_lds_reads<kBatch>();
+                add(w0);
+                chain_fence(s);
+                if (b + 2 < kBatches)
+                    read(w0, b + 2);
+                chain_fence(s);
+                if (b + 2 < kBatches)
+                    wait_lds_reads<kBatch>();
+                else
+                    wait_lds_reads<0>();
+                add(w1);
+                chain_fence(s);
+            }
+        }
+        __syncthreads();
+    };
+    static_assert(kDeepAhead == 3, "the pass loop below rotates three register sets");
+    for (int p0 = 0; p0 < npass; p0 += kDeepAhead) {
+        pass_step(p0, v[1]);
+        pass_step(p0 + 1, v[2]);
+        pass_step(p0 + 2, v[0]);
+    }
+    if (t < npx)
+        psum[m0 + t] = s;
+}
 
 __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, const ConvGeom g, int rb,
                                                                 int in_rows, int nthreads, const TensorQuant tq,
@@ -648,12 +952,19 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
         filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
         return;
     }
+    if (rb < 0) { // 1x1, stride 1, many channels, few pixels
+        if (in_rows == 8)
+            patch_sums_deep_body<8>(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8);
+        else
+            patch_sums_deep_body<16>(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8);
+        return;
+    }
     if (rb == 0) { // 1x1, stride 1: flat pixel list
         patch_sums_flat_body(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8, in_rows);
         return;
     }
     patch_sums_rows_body(x, g, rb, in_rows, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
-                         (int)gridDim.x - fw.blocks8, nthreads);
+                         (int)gridDim.x - fw.blocks8, nthreads, fw);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -1006,6 +1317,45 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const Ten
     return hipGetLastError();
 }
 
+// Band height for patch_sums_rows_body: the one with the least estimated time.  A block first copies its input rows
+// (all resident blocks of a CU share that CU's part of the memory bandwidth, ~17 bytes/ns with every CU copying), then
+// runs its chains: K dependent adds of ~2.75 ns each, one wavefront per 64 pixels, and a SIMD that holds several
+// such wavefronts interleaves them at no better than one add per ~1.9 ns, so lanes left idle by a thin band and
+// chain wavefronts that share a SIMD are what make deep layers slow.  Blocks beyond what the CUs hold at once
+// run as further rounds; the blocks that sum filter columns in the same launch (sum_blocks) count like the others.
+static void choose_band(const ConvGeom &g, int64_t row_bytes, int sum_blocks, int *rb_out, int *in_rows_out)
+{
+    const int cus = device_cus();
+    const double K = (double)g.KH * g.KW * g.C;
+    const int64_t lds_max = 160 * 1024;
+    double best = 0.0;
+    for (int cand = 1; cand <= g.OH && cand * g.OW <= 1024; ++cand) {
+        const int rows_needed = (cand - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+        const int64_t lds = rows_needed * row_bytes + (int64_t)(g.C + 4) * 4;
+        if (lds > lds_max)
+            break;
+        const int chains = cand * g.OW;
+        const int block_threads = chains <= 512 ? 512 : 1024;
+        int64_t per_cu = lds_max / lds;
+        if (per_cu > 2048 / block_threads)
+            per_cu = 2048 / block_threads;
+        const int64_t blocks = (int64_t)g.N * ((g.OH + cand - 1) / cand) + sum_blocks; // all of one LDS size
+        const int64_t rounds = (blocks + cus * per_cu - 1) / (cus * per_cu);
+        int64_t resident = (blocks + cus - 1) / cus;
+        if (resident > per_cu)
+            resident = per_cu;
+        const int64_t chain_waves = resident * ((chains + 63) / 64);
+        const double copy_ns = (double)(resident * lds) / 17.0;
+        const double chain_ns = K * 2.75 * (double)((chain_waves + 3) / 4);
+        const double t = (double)rounds * (copy_ns + chain_ns);
+        if (cand == 1 || t < best) {
+            best = t;
+            *rb_out = cand;
+            *in_rows_out = rows_needed;
+        }
+    }
+}
+
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
                              float *psum, hipStream_t stream, uint32_t *xq_fused, bool *fused,
                              const FilterJob *filter_job, bool *filter_done)
@@ -1032,9 +1382,19 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
         // 1x1, stride 1, no padding, and a band would hold few pixels (many channels): the flat-list variant
         const bool flat = g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 &&
                           rb * g.OW < 192;
+        if (!flat && rb > 0)
+            choose_band(g, row_bytes, (filter_job && filter_job->fsum && filter_job->filter) ? (int)blocks_for(g.Co, kFsCols) : 0,
+                        &rb, &in_rows);
+        // ... and with many channels and too few pixels to give every CU a workgroup of 64, the variant built around
+        // the chain of adds
+        const bool deep = flat && g.C >= 512 && g.M < (int64_t)64 * device_cus();
         if (flat) { // in_rows carries the pixels per workgroup: at least ~2 workgroups per CU where the layer allows
             rb = 0;
             in_rows = g.M >= 512 * kFlatPixels ? kFlatPixels : (g.M >= 512 * 128 ? 128 : 64);
+        }
+        if (deep) {
+            rb = -1;
+            in_rows = g.M >= (int64_t)2 * 16 * device_cus() ? 16 : 8;
         }
         if (rb > 0 || flat) {
             int threads = ((rb * g.OW + 63) / 64) * 64;
@@ -1047,7 +1407,9 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                                         (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0));
             if (fuse)
                 *fused = true;
-            size_t lds = flat ? (size_t)in_rows * kFlatPitch * 4 : (size_t)in_rows * row_bytes;
+            size_t lds = deep ? (size_t)deep_lds_bytes(in_rows)
+                              : flat ? (size_t)in_rows * kFlatPitch * 4
+                                     : (size_t)in_rows * row_bytes + (size_t)(g.C + 4) * 4; // + the pixel of zeros
             const int bands = flat ? 0 : (g.OH + rb - 1) / rb;
             const int64_t work_blocks = flat ? (g.M + in_rows - 1) / in_rows : (int64_t)g.N * bands;
             // the filter pre-pass rides along in the same launch (its workgroups want 512 or 1024 threads, so
@@ -1067,10 +1429,15 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 fw.n_col_tiles = plan.n_col_tiles;
                 fw.tq = filter_job->tq;
                 fw.wq = filter_job->wq;
-                fw.sum_blocks = (filter_job->fsum && filter_job->filter) ? (int)blocks_for(g.Co, 64) : 0;
+                fw.sum_blocks = (filter_job->fsum && filter_job->filter) ? (int)blocks_for(g.Co, kFsCols) : 0;
                 fw.fsum = filter_job->fsum;
                 block_threads = threads <= 512 ? 512 : 1024;
-                fw.blocks = fw.sum_blocks + (int)blocks_for(total, block_threads);
+                // A block of pack work would hold a patch-sum block's worth of LDS for nothing: with bands of rows
+                // (large LDS, most threads idle while the chains run) idle wavefronts of the patch-sum blocks pack,
+                // those on SIMDs that hold no chain, so at most three chain wavefronts per block.
+                if (!flat && rb * g.OW <= 3 * 64)
+                    fw.pack_total = total;
+                fw.blocks = fw.sum_blocks + (fw.pack_total > 0 ? 0 : (int)blocks_for(total, block_threads));
                 fw.blocks8 = (fw.blocks + 7) & ~7;
                 if (fw.sum_blocks && lds < (size_t)kFsLdsBytes)
                     lds = kFsLdsBytes;
@@ -1180,7 +1547,7 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
                               float *fsum, hipStream_t stream)
 {
     const int64_t total = (int64_t)plan.n_col_tiles * plan.fills * 64;
-    const int sum_blocks = (fsum && filter) ? (int)blocks_for(g.Co, 64) : 0;
+    const int sum_blocks = (fsum && filter) ? (int)blocks_for(g.Co, kFsCols) : 0;
     const size_t lds = sum_blocks ? kFsLdsBytes : 0;
     if (lds) {
         const hipError_t ea = set_max_dynamic_lds_once(reinterpret_cast<const void *>(filter_prep_kernel), kFsLdsBytes);
