@@ -75,8 +75,16 @@ LAYERS = [
 # scaled by what the same counter reads for --copy-calibration.  Not measured in the run that prints them: the
 # bench line says which profile they come from.
 PROFILED_TRAFFIC = {
-    "conv3x3_b64_56x56x64_to_64_s1_same": (2.000 * 13465.0 * 1024 + 1.000 * 72175.1 * 1024,
+    "conv3x3_b64_56x56x64_to_64_s1_same": (2.000 * 8034.0 * 1024 + 1.000 * 61573.5 * 1024,
                                            "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
+    "conv1x1_b64_112x112x32_to_192": (2.000 * 19020.5 * 1024 + 1.000 * 731723.0 * 1024,
+                                      "profiles/lutgemm_expand_conv1x1_b64_112x112x32_to_192.md"),
+    "conv1x1_b64_56x56x64_to_256": (2.000 * 8133.0 * 1024 + 1.000 * 253711.0 * 1024,
+                                    "profiles/lutgemm_expand_conv1x1_b64_56x56x64_to_256.md"),
+    "conv7x7s2_b64_224x224x3_to_64": (2.000 * 9278.5 * 1024 + 1.000 * 231414.8 * 1024,
+                                      "profiles/lutgemm_expand_conv7x7s2_b64_224x224x3_to_64.md"),
+    "conv1x1_b32_56x56x256_to_1024": (2.000 * 27862.1 * 1024 + 1.000 * 486248.0 * 1024,
+                                      "profiles/lutgemm_expand_conv1x1_b32_56x56x256_to_1024.md"),
     "dw3x3_b64_112x112x192_s1": (2.000 * 342889 * 1024 + 1.000 * 602112 * 1024,
                                  "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
     "dw3x3_b64_112x112x192_s2": (2.000 * 321245 * 1024 + 1.000 * 150528 * 1024,
