@@ -156,6 +156,24 @@ int axc_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc,
                       float input_min, float input_max, float filter_min, float filter_max,
                       float *output, void *workspace, size_t workspace_bytes, void *stream);
 
+/* The op followed by the tail of the Keras layer's call, bias_add and the activation of Conv.call
+ * (tf2/python/keras/layers/fake_approx_convolutional.py:261), fused into the op's store, for callers that hold the
+ * ranges themselves (fake-quantization variables fixed after training or calibration) and so have no use for
+ * the per-batch min / max pass of axc_fake_approx_conv2d.  Unlike that entry it does not fake-quantize: like the op,
+ * it expects tensors that already lie on their grids.  bias may be null (out_depth floats otherwise; in_depth for
+ * the depthwise variant); activation is AXC_ACT_*.  Results equal axc_conv2d_minmax / axc_depthwise_conv2d_minmax
+ * followed by `+ bias` and `max(x, 0)`, each rounded on its own. */
+int axc_conv2d_minmax_bias_act(const axc_table *table, const axc_conv2d_desc *desc,
+                               const float *input, const float *filter,
+                               float input_min, float input_max, float filter_min, float filter_max,
+                               const float *bias, int activation,
+                               float *output, void *workspace, size_t workspace_bytes, void *stream);
+int axc_depthwise_conv2d_minmax_bias_act(const axc_table *table, const axc_conv2d_desc *desc,
+                                         const float *input, const float *filter,
+                                         float input_min, float input_max, float filter_min, float filter_max,
+                                         const float *bias, int activation,
+                                         float *output, void *workspace, size_t workspace_bytes, void *stream);
+
 /* axc_conv2d_minmax for callers that cannot allocate or own a workspace (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose launcher allocates its
  * temporaries per call (approx_nn_conv_ops.cpp:590-613).  The workspace is a fixed array of

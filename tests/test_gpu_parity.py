@@ -428,6 +428,38 @@ def test_fake_approx_depthwise_layer_vs_composition(pkg, oracle, case):
     assert refimpl.linf_rel(y, y_ref) <= TOL
 
 
+@pytest.mark.parametrize("case", LAYER_CASES + DW_LAYER, ids=[str(i) for i in range(len(LAYER_CASES) + len(DW_LAYER))])
+def test_op_with_fused_bias_and_activation_vs_oracle(pkg, oracle, case):
+    """axc_conv2d_minmax_bias_act / axc_depthwise_conv2d_minmax_bias_act with ranges given by the caller: the oracle's
+    op on the same (raw) tensors and ranges, then bias_add and ReLU, each rounded on its own.  No fake quantization
+    here, unlike the layer entry points."""
+    xs, fs, strides, use_bias, activation, (lo, hi) = case
+    depthwise = fs[3] == 1 and fs[2] == xs[3] and case in DW_LAYER
+    rng = np.random.default_rng(xs[2] * 3 + fs[2])
+    x = rng.uniform(lo, hi, size=xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * 0.2).astype(np.float32)
+    nb = fs[2] if depthwise else fs[3]
+    bias = rng.uniform(-0.5, 0.5, size=nb).astype(np.float32) if use_bias else None
+    table = pkg.synth.table_noisy(5)
+    mm = (lo, hi, float(w.min()), float(w.max()))
+    op = pkg.ApproxConv2DWithMinMaxVars([1, strides[0], strides[1], 1], 8, table, "SAME", depthwise=depthwise)
+    dev = gpu_util.dev()
+    y = op(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev), *mm,
+           bias=torch.from_numpy(bias).to(dev) if use_bias else None, activation=activation).cpu().numpy()
+    fn = oracle.depthwise_conv2d if depthwise else oracle.conv2d_fast
+    rc, y_ref, _ = fn(table, x, w, *mm, strides=strides, padding="SAME", dilations=(1, 1))
+    assert rc == 0
+    if use_bias:
+        y_ref = (y_ref + bias).astype(np.float32)
+    if activation == "relu":
+        y_ref = np.maximum(y_ref, 0.0)
+    assert y.shape == y_ref.shape
+    assert refimpl.linf_rel(y, y_ref) <= TOL
+    if not use_bias and activation is None:   # then it is the plain op, bit for bit
+        y_plain = op(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev), *mm).cpu().numpy()
+        assert np.array_equal(y, y_plain)
+
+
 def test_fake_approx_conv2d_layer_strided_1x1_takes_minmax_of_the_whole_input(pkg, oracle):
     """A strided 1x1 layer reads a quarter of its input, but the layer's min / max are those of the whole tensor
     (fake_approx_convolutional.py:233-236): the extremes sit on pixels the filter never touches."""

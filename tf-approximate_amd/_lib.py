@@ -59,6 +59,9 @@ SYMBOLS = [
     ("axc_depthwise_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
+    ("axc_conv2d_minmax_bias_act", ctypes.c_int, [_vp, _desc, _vp, _vp, _f, _f, _f, _f, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
+    ("axc_depthwise_conv2d_minmax_bias_act", ctypes.c_int,
+     [_vp, _desc, _vp, _vp, _f, _f, _f, _f, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),
     ("axc_conv2d_static_workspace_limit", ctypes.c_int, [ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax_static", ctypes.c_int, [_vp, _desc, _vp, _vp, _f, _f, _f, _f, _vp, _vp]),
     ("axc_fake_approx_conv2d", ctypes.c_int, [_vp, _desc, _vp, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _vp]),

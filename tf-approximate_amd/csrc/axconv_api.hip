@@ -1066,6 +1066,28 @@ int axc_conv2d_minmax(const axc_table *table, const axc_conv2d_desc *desc, const
                      filter_max, output, nullptr, workspace, workspace_bytes, stream);
 }
 
+int axc_conv2d_minmax_bias_act(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                               const float *filter, float input_min, float input_max, float filter_min,
+                               float filter_max, const float *bias, int activation, float *output, void *workspace,
+                               size_t workspace_bytes, void *stream)
+{
+    if (!output)
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    return run_dense(table, desc, input, filter, nullptr, nullptr, 0, input_min, input_max, filter_min,
+                     filter_max, output, nullptr, workspace, workspace_bytes, stream, false, bias, activation);
+}
+
+int axc_depthwise_conv2d_minmax_bias_act(const axc_table *table, const axc_conv2d_desc *desc, const float *input,
+                                         const float *filter, float input_min, float input_max, float filter_min,
+                                         float filter_max, const float *bias, int activation, float *output,
+                                         void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!output)
+        return fail(AXC_INVALID_ARGUMENT, "null tensor pointer");
+    return run_depthwise(table, desc, input, filter, input_min, input_max, filter_min, filter_max, output,
+                         nullptr, workspace, workspace_bytes, stream, false, bias, activation);
+}
+
 int axc_conv2d_static_workspace_limit(size_t *bytes)
 {
     if (!bytes)

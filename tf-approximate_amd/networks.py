@@ -9,7 +9,8 @@ forward pass from layer lists, random He-normal weights and synthetic inputs:
     resnet50       ResNet-50 shaped: 7x7/2 stem, bottlenecks 1x1 / 3x3 / 1x1, stage widths 256/512/1024/2048
     inverted_residual  MobileNetV2-style block: 1x1 expand (x6), depthwise 3x3 (stride 1 or 2), 1x1 project
 
-Only the convolutions run through the library; ReLU, residual adds and the max-pool are torch glue.  The
+Only the convolutions run through the library (with the ReLU that directly follows one fused into its store);
+residual adds with their ReLU and the max-pool are torch glue.  The
 min/max of every layer input and filter are taken from the tensors in a calibration pass (the Keras wrapper's
 policy) and then held fixed, so the timed pass has no host synchronisation.
 """
@@ -43,11 +44,12 @@ class ApproxNetwork:
     """A forward pass described as a small program over named tensors:
     ("conv", dst, src, ConvSpec) | ("add_relu", dst, a, b) | ("maxpool", dst, src)"""
 
-    def __init__(self, program, input_shape, table, seed=0, device="cuda:0", fused_layers=False):
+    def __init__(self, program, input_shape, table, seed=0, device="cuda:0", fused_layers=False, fuse_relu=True):
         """fused_layers: run every convolution, dense or depthwise, through the layer entry point (min/max of each batch and
         fake quantization computed on the device, ReLU fused), as the reference's Keras layer does per call;
         otherwise ranges come from a calibration pass and the plain op runs."""
         self.fused_layers = fused_layers
+        self.fuse_relu = fuse_relu   # calibrated mode: conv + ReLU as one call (axc_conv2d_minmax_bias_act)
         self.program = program
         self.input_shape = tuple(input_shape)
         self.device = torch.device(device)
@@ -96,13 +98,17 @@ class ApproxNetwork:
                     lo, hi = torch.aminmax(src)
                     wlo, whi = torch.aminmax(w)
                     self.ranges[i] = (float(lo), float(hi), float(wlo), float(whi))
-                y = self.ops[i](src, w, *self.ranges[i])
-                if trace is not None:
-                    trace.append((spec, src.cpu().numpy(), w.cpu().numpy(), self.ranges[i], y.cpu().numpy()))
+                if trace is not None or not self.fuse_relu:
+                    y = self.ops[i](src, w, *self.ranges[i])
+                    if trace is not None:
+                        trace.append((spec, src.cpu().numpy(), w.cpu().numpy(), self.ranges[i], y.cpu().numpy()))
+                    y = torch.relu_(y) if spec.relu else y
+                else:   # a ReLU that directly follows the convolution goes into its store
+                    y = self.ops[i](src, w, *self.ranges[i], activation="relu" if spec.relu else None)
                 macs += spec.macs(y.shape[1], y.shape[2], y.shape[0])
-                t[dst] = torch.relu_(y) if spec.relu else y
-            elif kind == "add_relu":
-                t[dst] = torch.relu_(t[step[2]] + t[step[3]])
+                t[dst] = y
+            elif kind == "add_relu":   # the first operand is a convolution's fresh output: added to in place
+                t[dst] = torch.relu_(t[step[2]].add_(t[step[3]]))
             elif kind == "maxpool":
                 nchw = t[step[2]].permute(0, 3, 1, 2)
                 t[dst] = torch.nn.functional.max_pool2d(nchw, 3, 2, 1).permute(0, 2, 3, 1).contiguous()

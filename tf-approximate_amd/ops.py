@@ -189,8 +189,35 @@ class ApproxConv2DWithMinMaxVars:
                       _stream_ptr(input.device)))
         return out
 
-    def __call__(self, input, filter, input_min, input_max, filter_min, filter_max):
-        return self._run(input, filter, (input_min, input_max, filter_min, filter_max), False)
+    def __call__(self, input, filter, input_min, input_max, filter_min, filter_max, bias=None, activation=None):
+        """The op.  With `bias` and / or `activation` ("relu"): the op followed by bias_add and the activation, fused
+        into its store (the tail of the Keras layer's call, fake_approx_convolutional.py:261)."""
+        if bias is None and activation is None:
+            return self._run(input, filter, (input_min, input_max, filter_min, filter_max), False)
+        if activation not in (None, "relu"):
+            raise InvalidArgumentError("activation must be None or 'relu'")
+        lib = _lib.load()
+        input = _require_device_f32(input, "input")
+        filter = _require_device_f32(filter, "filter")
+        desc = self._desc(input, filter)
+        dims = conv2d_geometry(desc)
+        out_shape = self._out_shape(dims)
+        if bias is not None:
+            bias = _require_device_f32(bias, "bias")
+            if bias.numel() != out_shape[3]:
+                raise InvalidArgumentError("bias must have one value per output channel")
+        nbytes = ctypes.c_size_t()
+        ws_fn = lib.axc_depthwise_conv2d_workspace_bytes if self.depthwise else lib.axc_conv2d_workspace_bytes
+        _check(ws_fn(ctypes.byref(desc), ctypes.byref(nbytes)))
+        ws = _workspace(input.device, nbytes.value)
+        out = torch.empty(out_shape, dtype=torch.float32, device=input.device)
+        fn = lib.axc_depthwise_conv2d_minmax_bias_act if self.depthwise else lib.axc_conv2d_minmax_bias_act
+        with torch.cuda.device(input.device):
+            _check(fn(self.table.handle, ctypes.byref(desc), input.data_ptr(), filter.data_ptr(),
+                      *[_scalar(m) for m in (input_min, input_max, filter_min, filter_max)],
+                      bias.data_ptr() if bias is not None else None, 1 if activation == "relu" else 0,
+                      out.data_ptr(), ws.data_ptr(), ws.numel(), _stream_ptr(input.device)))
+        return out
 
     def accumulators(self, input, filter, input_min, input_max, filter_min, filter_max):
         """int32 sums of table entries before the epilogue (parity entry point)."""
