@@ -100,6 +100,7 @@ struct DenseParams {
     const LayerQuant *lq_dev;    // not null: epilogue constants come from here instead of the four floats above
     const float *bias;           // not null: added to every output column after the epilogue
     int relu;                    // 1: max(x, 0) last
+    int stagger_sleeps;          // s_sleep(127) periods by which every second group of workgroups starts late (0: none)
 };
 
 struct DepthwiseParams {
@@ -116,6 +117,7 @@ struct DepthwiseParams {
     const LayerQuant *lq_dev;    // not null (layer entry point): input quantization and epilogue constants from here
     const float *bias;           // not null: added per channel after the epilogue
     int relu;                    // 1: max(x, 0) last
+    int stagger_sleeps;          // s_sleep(127) periods by which every second group of workgroups starts late (0: none)
 };
 
 // Row permutation of the expanded table: logical activation code a lives in physical row

@@ -158,6 +158,9 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     // at about the same time) meet in one L2.
     const int G = (int)gridDim.x;
     const int wg = (G & 7) == 0 ? ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
+    if (p.stagger_sleeps && ((wg / nct_v) & 1)) // every second group of workgroups (one row tile's column tiles) starts late
+        for (int i = 0; i < p.stagger_sleeps; ++i)
+            __builtin_amdgcn_s_sleep(127);
     int prev_rt = -1;
     bool rvalid[DenseCfg<NT>::R];    // this lane's pixel exists
     uint32_t nr = 0;                 // pixels of this lane whose wavefront row exists (a prefix; wave-uniform)
@@ -378,11 +381,15 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
 
         // The phases add whole dwords (two 16-bit table entries) into the accumulator of the even column and the
         // high entry alone into that of the odd column: even = sum(lo) + 65536 * sum(hi) modulo 2^32.
+        // Subtracting a multiple of 65536 changes the high half only: one 16-bit subtract (high half of the even
+        // accumulator minus low half of the odd one, written back into the high half, low half kept).
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int j = 0; j < NT; j += 2)
-                acc[r][j] = (int32_t)((uint32_t)acc[r][j] - ((uint32_t)acc[r][j + 1] << 16));
+                __asm__("v_sub_u16_sdwa %0, %0, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1 src1_sel:WORD_0"
+                        : "+v"(acc[r][j])
+                        : "v"(acc[r][j + 1]));
 
         // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----
         // A lane holds NT consecutive columns of its pixel: stored as they are, one instruction would touch 64
@@ -421,6 +428,10 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 t3q[j] = OUT_I32 ? 0.0f : __fmul_rn(e_m1, p.fsum[c]);
                 biasq[j] = (!OUT_I32 && p.bias) ? p.bias[c] : 0.0f;
             }
+            // bias and ReLU are wave-uniform run-time switches: one copy of the store loop per combination, chosen
+            // once, instead of two selects per output element
+            auto store_rows = [&](auto has_bias_t, auto has_relu_t) {
+            constexpr bool kBias = decltype(has_bias_t)::value, kRelu = decltype(has_relu_t)::value;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (r >= (int)nr_s)
@@ -453,9 +464,9 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             float v = __fsub_rn(__fadd_rn(__uint_as_float(d[j]), t3q[j]), e_km);
-                            if (p.bias)
+                            if (kBias)
                                 v = __fadd_rn(v, biasq[j]);
-                            d[j] = __float_as_uint(p.relu ? fmaxf(v, 0.0f) : v);
+                            d[j] = __float_as_uint(kRelu ? fmaxf(v, 0.0f) : v);
                         }
                     }
                     if (pix < nvalid && colq < g.Co) {
@@ -468,6 +479,17 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                     }
                 }
             }
+            };
+            using yes = std::true_type;
+            using no = std::false_type;
+            if (OUT_I32 || (!p.bias && !p.relu))
+                store_rows(no(), no());
+            else if (p.bias && p.relu)
+                store_rows(yes(), yes());
+            else if (p.bias)
+                store_rows(yes(), no());
+            else
+                store_rows(no(), yes());
             continue;
         }
 #pragma unroll
