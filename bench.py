@@ -259,6 +259,11 @@ def sampled_oracle_check(oracle, table, op, xd, fd, strides, depthwise, y, n_sam
     return bit_exact, linf
 
 
+def dense_kernel_name(kernels_ms):
+    """The LUT-GEMM kernel a dense layer ran: out of pre-expanded rows, or expanding inside every tile."""
+    return "lutgemm_px" if "lutgemm_px" in kernels_ms else "lutgemm_expand"
+
+
 def measure_layer(pkg, ops, oracle, ceil, spec, steps=None, preroll_s=0.08):
     config, name, xs, fs, strides, depthwise, codes, tkind = spec
     table = make_table(pkg.synth, tkind)
@@ -271,7 +276,7 @@ def measure_layer(pkg, ops, oracle, ceil, spec, steps=None, preroll_s=0.08):
     N, OH, OW, Cout = y.shape
     taps_c = fs[0] * fs[1] * (1 if depthwise else fs[2])
     lookups = N * OH * OW * Cout * taps_c
-    main = "depthwise_lut" if depthwise else "lutgemm_expand"
+    main = "depthwise_lut" if depthwise else dense_kernel_name(kms)
     kernel_ms = kms[main]
     rec = {"config": config, "layer": name, "input": list(xs), "filter": list(fs), "strides": list(strides),
            "codes": codes, "table": tkind, "M": N * OH * OW, "K": taps_c, "N": Cout, "lookups": lookups,
@@ -422,7 +427,7 @@ def main():
     lookups = n * oh * ow * co * taps_c
     gmacs = lookups / (ms_per_step * 1e-3) / 1e9
 
-    main_kernel = "depthwise_lut" if depthwise else "lutgemm_expand"
+    main_kernel = "depthwise_lut" if depthwise else dense_kernel_name(kms)
     main_ms = kms[main_kernel]
     achieved = lookups / (main_ms * 1e-3)
     ceil = Ceilings(ops)

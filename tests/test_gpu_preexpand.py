@@ -1,0 +1,149 @@
+"""The dense kernel that reads pre-expanded rows (lutgemm_px_kernel.hip) against the oracle.
+
+The planner only picks it for layers with many output pixels, so the small cases here force it through
+axc_set_preexpand(1); every case also checks, from the library's own kernel timers, that this kernel is the one that
+ran.  Shapes cover one and many fills, odd and even fill counts (the two ways a tile hands LDS buffer 0 to the next
+tile), several tiles per workgroup, ragged row tiles, column counts that are not multiples of 16 or of 4, strides,
+dilation, padding taps, the layer entry point and the codes entry point."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_util
+import refimpl
+
+pytestmark = pytest.mark.gpu
+
+MM = (-1.0, 1.0, -0.5, 0.5)
+
+CASES = [
+    # input, filter, strides, dilations, padding
+    ((2, 9, 9, 8), (1, 1, 8, 16), (1, 1), (1, 1), "SAME"),        # one fill
+    ((2, 9, 9, 8), (3, 3, 8, 16), (1, 1), (1, 1), "SAME"),        # nine fills (odd), padding taps
+    ((1, 12, 11, 16), (3, 3, 16, 24), (1, 1), (1, 1), "SAME"),    # 18 fills (even), two column tiles
+    ((3, 17, 13, 16), (3, 3, 16, 30), (2, 2), (1, 1), "VALID"),   # columns not a multiple of four: untransposed store
+    ((2, 20, 20, 24), (5, 5, 24, 7), (1, 1), (1, 1), "SAME"),     # fewer than 16 columns
+    ((2, 21, 19, 6), (3, 3, 6, 20), (1, 2), (2, 1), "SAME"),      # 6 channels in two quads, dilation, mixed strides
+    ((1, 40, 40, 32), (1, 1, 32, 100), (1, 1), (1, 1), "SAME"),   # seven column tiles: two blocks of the tile order
+    ((70, 9, 9, 8), (3, 3, 8, 24), (2, 2), (1, 1), "VALID"),      # many small images
+    ((9, 60, 60, 8), (1, 1, 8, 160), (1, 1), (1, 1), "SAME"),     # 8 row tiles x 10 column tiles
+]
+
+
+def _ran_px(ops):
+    prof = ops.profile_read()
+    return "lutgemm_px" in prof and "lutgemm_expand" not in prof
+
+
+@pytest.fixture()
+def forced(pkg):
+    from tf_approximate_amd import ops
+    ops.set_preexpand(1)
+    ops.profile_enable(True)
+    ops.profile_reset()
+    yield ops
+    ops.profile_enable(False)
+    ops.set_preexpand(0)
+
+
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_preexpanded_rows_vs_oracle(pkg, oracle, forced, case):
+    xs, fs, strides, dil, padding = case
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=len(str(case)))
+    table = pkg.synth.table_random(9) if xs[0] % 2 else pkg.synth.table_asymmetric()
+    y, acc = gpu_util.run_op(pkg, table, x, f, MM, strides, padding, dil)
+    assert _ran_px(forced), case
+    rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *MM, strides=strides, padding=padding, dilations=dil, threads=8)
+    assert rc == 0
+    assert np.array_equal(acc, acc_ref), case
+    assert refimpl.linf_rel(y, y_ref) <= 1e-5, case
+
+
+def test_many_tiles_per_workgroup_match_the_other_kernel(pkg, forced):
+    """1x1 32 -> 192 on 8 x 112 x 112: 25 row tiles x 12 column tiles, more than one tile per workgroup, one fill each
+    (every tile's fill is fetched by the tile before it).  Compared bit for bit with the kernel that expands inside
+    every tile, which the full-size tests pin against the oracle."""
+    xs, fs = (8, 112, 112, 32), (1, 1, 32, 192)
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=4)
+    table = pkg.synth.table_random(3)
+    y, acc = gpu_util.run_op(pkg, table, x, f, MM)
+    assert _ran_px(forced)
+    forced.set_preexpand(-1)
+    forced.profile_reset()
+    y0, acc0 = gpu_util.run_op(pkg, table, x, f, MM)
+    assert not _ran_px(forced)
+    assert np.array_equal(acc, acc0)
+    assert np.array_equal(y.view(np.uint32), y0.view(np.uint32))
+
+
+def test_layer_entry_point_on_preexpanded_rows(pkg, oracle, forced):
+    """Per-batch min/max, fake quantization, bias and ReLU around the pre-expanded kernel."""
+    rng = np.random.default_rng(77)
+    xs, fs = (2, 18, 18, 16), (3, 3, 16, 40)
+    x = rng.uniform(-2.0, 1.0, size=xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * 0.3).astype(np.float32)
+    bias = rng.uniform(-1, 1, size=fs[3]).astype(np.float32)
+    table = pkg.synth.table_noisy(5)
+    dev = gpu_util.dev()
+    layer = pkg.FakeApproxConv2D((1, 1), table, "SAME", activation="relu")
+    y = layer(torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev), torch.from_numpy(bias).to(dev)).cpu().numpy()
+    assert _ran_px(forced)
+    r = (float(x.min()), float(x.max()), float(w.min()), float(w.max()))
+    fq = pkg.fake_quant.fake_quant_with_min_max_vars
+    rc, y_ref, _ = oracle.conv2d_fast(table, fq(x, r[0], r[1]), fq(w, r[2], r[3]), *r, strides=(1, 1), padding="SAME")
+    assert rc == 0
+    y_ref = np.maximum((y_ref + bias).astype(np.float32), 0.0)
+    assert refimpl.linf_rel(y, y_ref) <= 1e-5
+
+
+def test_workspace_without_room_for_the_rows_still_serves(pkg, forced):
+    """The workspace query counts the pre-expanded rows; the allocation-free entry point has 32 MiB and runs a layer
+    whose rows alone take 128 MiB without them - same bits."""
+    from tf_approximate_amd import _lib, ops
+    lib = _lib.load()
+    xs, fs = (16, 28, 28, 256), (1, 1, 256, 1024)
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=21)
+    dev = gpu_util.dev()
+    xd, fd = torch.from_numpy(x).to(dev), torch.from_numpy(f).to(dev)
+    table = ops.TruthTable(pkg.synth.table_random(1))
+    desc = ops.make_desc(xs, fs, [1, 1, 1, 1], "SAME")
+    nbytes = ctypes.c_size_t()
+    assert lib.axc_conv2d_workspace_bytes(ctypes.byref(desc), ctypes.byref(nbytes)) == 0
+    assert nbytes.value > 128 << 20
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+    shape = (xs[0], xs[1], xs[2], fs[3])
+    want = torch.full(shape, float("nan"), dtype=torch.float32, device=dev)
+    got = torch.full(shape, float("nan"), dtype=torch.float32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    assert lib.axc_conv2d_minmax(table.handle, ctypes.byref(desc), xd.data_ptr(), fd.data_ptr(), *MM, want.data_ptr(),
+                                 ws.data_ptr(), ws.numel(), stream) == 0, lib.axc_last_error()
+    torch.cuda.synchronize()
+    assert _ran_px(forced)
+    forced.profile_reset()
+    assert lib.axc_conv2d_minmax_static(table.handle, ctypes.byref(desc), xd.data_ptr(), fd.data_ptr(), *MM,
+                                        got.data_ptr(), stream) == 0, lib.axc_last_error()
+    torch.cuda.synchronize()
+    assert not _ran_px(forced)
+    assert np.array_equal(want.cpu().numpy().view(np.uint32), got.cpu().numpy().view(np.uint32))
+
+
+def test_planner_picks_preexpanded_rows_for_many_pixels_only(pkg):
+    """Without forcing: the north-star layer runs out of pre-expanded rows, a 14 x 14 layer of the same filter does not."""
+    from tf_approximate_amd import ops
+    table = pkg.synth.table_random(2)
+    dev = gpu_util.dev()
+    ops.set_preexpand(0)
+    ops.profile_enable(True)
+    try:
+        for xs, expect in (((64, 56, 56, 64), True), ((4, 14, 14, 64), False)):
+            x = torch.zeros(xs, dtype=torch.float32, device=dev)
+            f = torch.zeros((3, 3, 64, 64), dtype=torch.float32, device=dev)
+            op = pkg.ApproxConv2DWithMinMaxVars([1, 1, 1, 1], 8, table, "SAME")
+            ops.profile_reset()
+            op(x, f, *MM)
+            torch.cuda.synchronize()
+            assert _ran_px(ops) == expect, xs
+    finally:
+        ops.profile_enable(False)

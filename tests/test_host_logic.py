@@ -141,7 +141,13 @@ def test_workspace_sizes(ops, lib):
     assert rc == 0
     xq = 64 * 56 * 56 * 64            # one byte per activation
     psum = 64 * 56 * 56 * 4
-    assert xq + psum < n < xq + psum + (1 << 20)
+    rows = 4 * (9 * 16 // 2) * 65536  # pre-expanded rows: 4 column tiles x 72 fills (pairs of channel quads) x 64 KiB
+    assert xq + psum + rows < n < xq + psum + rows + (1 << 20)
+    assert lib.axc_set_preexpand(-1) == 0
+    rc, n = _ws(lib, desc)
+    assert lib.axc_set_preexpand(0) == 0
+    assert rc == 0 and xq + psum < n < xq + psum + (1 << 20)
+    assert lib.axc_set_preexpand(2) == 1
     rc, n0 = _ws(lib, ops.make_desc((0, 56, 56, 64), (3, 3, 64, 64), (1, 1, 1, 1), "SAME"))
     assert rc == 0 and n0 == 0        # empty output: nothing to do (approx_nn_conv_ops.cpp:449)
     rc, nd = _ws(lib, ops.make_desc((2, 8, 8, 6), (3, 3, 6, 1), (1, 1, 1, 1), "SAME"), depthwise=True)

@@ -111,6 +111,57 @@ def test_every_path_waits_for_what_it_uses(nt, buf):
     assert counts == [8 * r for r in range(rows + 1)]
 
 
+@pytest.mark.parametrize("buf", [0, 1])
+def test_every_path_of_the_pre_expanded_phase_waits_for_what_it_uses(buf):
+    """The phase that reads pre-expanded fills: 16 lookups per pixel (two activation dwords), eight loads that copy
+    the next fill into LDS, two activation loads per pixel."""
+    gen = _generator()
+    prog = _instructions(gen.emit_px(buf))
+    paths = _paths(prog)
+    assert len(paths) == 9               # 0 pixels, or the last pixel is pixel 0 .. 7
+    for trace in paths:
+        _check_path(trace)
+        assert sum(1 for t in trace if t.startswith("buffer_load_dwordx4") and t.endswith(" lds")) == 8
+        assert sum(1 for t in trace if t.startswith("buffer_load_dword ")) == 16
+        # the LDS destination register is written one instruction ahead of the load that uses it, at least
+        for i, t in enumerate(trace):
+            if t.startswith("buffer_load_dwordx4"):
+                assert trace[i - 2].startswith("s_add_u32 m0,") and not trace[i - 1].startswith("s_add_u32 m0,")
+    counts = sorted(sum(1 for t in trace if t.startswith("ds_read_b128")) for trace in paths)
+    assert counts == [16 * r for r in range(9)]
+    # buffer 1 is addressed through the instruction offset, buffer 0 without one; the fill lands in the other buffer
+    reads = [t for t in max(paths, key=len) if t.startswith("ds_read_b128")]
+    assert all(t.endswith("offset:65521") for t in reads) if buf else all("offset" not in t for t in reads)
+    dests = sorted(int(t.split(",")[-1]) for t in max(paths, key=len) if t.startswith("s_add_u32 m0,"))
+    assert dests == [(1 - buf) * 65536 + j * 1024 for j in range(8)]
+
+
+def test_every_accumulator_gets_its_share_of_a_pre_expanded_fill():
+    """A pre-expanded fill holds 8 input channels for each of 16 columns: every accumulator of every pixel receives
+    eight entries, even columns from whole dwords, odd columns from high halves, and every landed dword is used once
+    whole and once for its high half per unit (two units per pixel)."""
+    gen = _generator()
+    path = max(_paths(_instructions(gen.emit_px(0))), key=len)
+    adds, uses = {}, {}
+    for text in path:
+        if text.startswith("v_add_u32_sdwa") or text.startswith("v_add3_u32"):
+            toks = TOKEN.findall(text)
+            dst, sources = toks[0], toks[2:]
+            assert toks[1] == dst and dst.startswith("%[c")
+            high = "WORD_1" in text
+            adds.setdefault(dst, []).extend([high] * len(sources))
+            for src in sources:
+                uses.setdefault(src, []).append(high)
+    assert len(adds) == 8 * 16
+    for r in range(8):
+        for j in range(16):
+            kinds = adds["%%[c%d_%d]" % (r, j)]
+            assert len(kinds) == 8 and all(k == bool(j & 1) for k in kinds)
+    assert len(uses) == 32
+    for src, kinds in uses.items():
+        assert sorted(kinds) == [False] * 16 + [True] * 16, src
+
+
 def test_the_model_notices_a_missing_wait():
     """The checker itself: dropping one s_waitcnt from a path must be reported."""
     gen = _generator()

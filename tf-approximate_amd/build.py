@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libaxconv_hip.so")
-SOURCES = ["axconv_api.hip", "lutgemm_kernel.hip", "prepass_kernels.hip", "depthwise_kernel.hip"]
+SOURCES = ["axconv_api.hip", "lutgemm_kernel.hip", "lutgemm_px_kernel.hip", "prepass_kernels.hip", "depthwise_kernel.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -342,13 +342,25 @@ std::atomic<int> g_forced_nt{[] {
     return (v == 16 || v == 32 || v == 64) ? v : 0;
 }()};
 
+// Pre-expanded rows (lutgemm_px_kernel.hip): 0 = the planner decides, 1 = every layer that can run that way does,
+// -1 = never.  Set by axc_set_preexpand; AXC_PREEXPAND gives the initial value, read once when the library is loaded.
+std::atomic<int> g_px_mode{[] {
+    const char *env = std::getenv("AXC_PREEXPAND");
+    const int v = env ? std::atoi(env) : 0;
+    return (v == 1 || v == -1) ? v : 0;
+}()};
+constexpr size_t kPxMaxBytes = (size_t)192 << 20;   // most memory a layer's pre-expanded rows may take
+
 // Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
 // Derive cost per fill is constant; lookup cost per fill grows with the wavefront-rows a SIMD carries.
-DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt)
+DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
 {
     DensePlan best{};
     double best_cost = 1e300;
     const int taps = g.KH * g.KW;
+    const bool px_possible = (g.C4 & 1) == 0 &&
+                             (size_t)((g.Co + 15) / 16) * (size_t)(taps * g.C4 / 2) * 65536 <= kPxMaxBytes;
+    const bool want_px = px_mode > 0 && px_possible && (forced_nt == 0 || forced_nt == 16);
     for (int nt : {16, 32, 64}) {
         if (forced_nt == 16 || forced_nt == 32 || forced_nt == 64) {
             if (nt != forced_nt)
@@ -381,6 +393,8 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt)
             // Splitting K over tiles keeps the tiles tall (many lookups per expanded fill) when M alone does not
             // give every CU a tile; the int32 partial sums then cost one more pass over (k_splits + 1) outputs.
             for (int ks : {1, 2, 3, 4, 6, 8, 12, 16}) {
+                if (want_px && (ks > 1 || nt != 16))
+                    break;  // pre-expanded rows are asked for wherever they are possible: 16 columns, whole K
                 const int fps = (fills + ks - 1) / ks;
                 if (ks > 1 && (fps < 8 || (int64_t)(ks - 1) * fps >= fills))
                     continue;
@@ -404,6 +418,17 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt)
             }
         }
     }
+    // Pre-expanded rows: 16-column tiles over the whole K, channel quads in pairs.  They cost 512 bytes of memory per
+    // filter element, written once per call (one more launch: ~7 us, then ~3 TB/s) and read once per XCD; the lookup
+    // kernel then runs about an eighth faster (measured: 11-14 % at ~24 T lookups/s).  Worth it with many output
+    // pixels per filter element.
+    best.px = 0;
+    const size_t px_bytes = (size_t)best.n_col_tiles * (size_t)(best.fills / 2) * 65536;
+    if (px_mode >= 0 && best.nt == 16 && best.k_splits == 1 && (g.C4 & 1) == 0 && px_bytes <= kPxMaxBytes) {
+        const double lookups = (double)g.M * (double)best.fills * 4.0 * (double)best.n_col_tiles * 16.0;
+        const double gain_s = 0.11 * lookups / 24e12, cost_s = 7e-6 + (double)px_bytes / 3e12;
+        best.px = (px_mode > 0 || gain_s > cost_s) ? 1 : 0;
+    }
     return best;
 }
 
@@ -412,23 +437,25 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt)
 DensePlan make_plan(const ConvGeom &g, int cus)
 {
     struct Key {
-        int taps, c4, co, cus, forced;
+        int taps, c4, co, cus, forced, px_mode;
         int64_t m;
         bool operator<(const Key &o) const
         {
-            return std::tie(taps, c4, co, cus, forced, m) < std::tie(o.taps, o.c4, o.co, o.cus, o.forced, o.m);
+            return std::tie(taps, c4, co, cus, forced, px_mode, m) <
+                   std::tie(o.taps, o.c4, o.co, o.cus, o.forced, o.px_mode, o.m);
         }
     };
     static std::mutex mu;
     static std::map<Key, DensePlan> cache;
-    const Key key{g.KH * g.KW, g.C4, g.Co, cus, g_forced_nt.load(std::memory_order_relaxed), g.M};
+    const Key key{g.KH * g.KW, g.C4, g.Co, cus, g_forced_nt.load(std::memory_order_relaxed),
+                  g_px_mode.load(std::memory_order_relaxed), g.M};
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = cache.find(key);
         if (it != cache.end())
             return it->second;
     }
-    const DensePlan plan = compute_plan(g, cus, key.forced);
+    const DensePlan plan = compute_plan(g, cus, key.forced, key.px_mode);
     std::lock_guard<std::mutex> lock(mu);
     if (cache.size() >= 4096)
         cache.clear();
@@ -439,7 +466,9 @@ DensePlan make_plan(const ConvGeom &g, int cus)
 inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct DenseWorkspace {
-    size_t sub_off, xq_off, psum_off, wq_off, fsum_off, layer_off, part_off, total;
+    size_t sub_off, xq_off, psum_off, wq_off, fsum_off, layer_off, part_off, px_off, px_bytes;
+    size_t total;        // everything, the pre-expanded rows (last) included
+    size_t total_no_px;  // what a launch needs that does without them
 };
 
 // sub_bytes: room for the pixels a strided 1x1 filter reads, gathered into a dense tensor (see prepare_dense)
@@ -457,6 +486,10 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan, size_t 
     w.part_off = off;   // int32 partial sums of the K splits
     if (plan.k_splits > 1)
         off += align_up((size_t)plan.k_splits * (size_t)g.M * g.Co * 4);
+    w.total_no_px = off;
+    w.px_off = off;
+    w.px_bytes = plan.px ? (size_t)plan.n_col_tiles * (size_t)(plan.fills / 2) * 65536 : 0;
+    off += align_up(w.px_bytes);
     w.total = off;
     return w;
 }
@@ -553,7 +586,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
                                 stream));
         return AXC_OK;
     }
-    if (workspace_bytes < pd.ws.total || (!workspace && pd.ws.total))
+    // a workspace without room for the pre-expanded rows still serves: the layer then runs without them
+    const bool use_px = pd.plan.px && workspace_bytes >= pd.ws.total;
+    if (workspace_bytes < pd.ws.total_no_px || (!workspace && pd.ws.total_no_px))
         return fail(AXC_INVALID_ARGUMENT, "workspace too small (see axc_conv2d_workspace_bytes)");
     if (((uintptr_t)workspace & 255) != 0)
         return fail(AXC_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
@@ -635,6 +670,15 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         p.step_oh = (int)((step % ohow) / g.OW);
         p.step_ow = (int)(step % g.OW);
     }
+    p.px_rows = nullptr;
+    p.px_bytes = 0;
+    if (use_px) {
+        ProfScope ps("px_expand_rows", stream);
+        uint16_t *rows = reinterpret_cast<uint16_t *>(ws + pd.ws.px_off);
+        AXC_HIP(launch_px_expand_rows(wq, table->dev_tableT, pd.plan, rows, stream));
+        p.px_rows = rows;
+        p.px_bytes = (uint32_t)pd.ws.px_bytes;
+    }
     p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
     p.wq_bytes = (uint32_t)((size_t)pd.plan.n_col_tiles * pd.plan.fills * 128);
     {
@@ -664,6 +708,11 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         }
         ProfScope ps("splitk_epilogue", stream);
         AXC_HIP(launch_splitk_epilogue(p, part, out_f, out_i, stream));
+        return AXC_OK;
+    }
+    if (use_px) {
+        ProfScope ps("lutgemm_px", stream);
+        AXC_HIP(launch_dense_px(p, out_i != nullptr, stream));
         return AXC_OK;
     }
     {
@@ -1060,6 +1109,14 @@ int axc_set_tile_columns(int columns)
     return AXC_OK;
 }
 
+int axc_set_preexpand(int mode)
+{
+    if (mode < -1 || mode > 1)
+        return fail(AXC_INVALID_ARGUMENT, "preexpand mode must be 0 (planner's choice), 1 (whenever possible) or -1 (never)");
+    g_px_mode.store(mode, std::memory_order_relaxed);
+    return AXC_OK;
+}
+
 int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes)
 {
     if (!bytes)
@@ -1123,10 +1180,10 @@ int axc_conv2d_minmax_static(const axc_table *table, const axc_conv2d_desc *desc
     int rc = prepare_dense(desc, &pd);
     if (rc != AXC_OK)
         return rc;
-    if (pd.ws.total > kStaticScratchBytes) {
+    if (pd.ws.total_no_px > kStaticScratchBytes) {
         char msg[200];
         snprintf(msg, sizeof(msg), "layer needs %zu bytes of workspace, the static workspace holds %zu: use "
-                 "axc_conv2d_minmax with a caller-owned workspace", pd.ws.total, kStaticScratchBytes);
+                 "axc_conv2d_minmax with a caller-owned workspace", pd.ws.total_no_px, kStaticScratchBytes);
         return fail(AXC_INVALID_ARGUMENT, msg);
     }
     void *ws = nullptr;

@@ -48,6 +48,7 @@ struct DensePlan {
     int k_splits;          // tiles along K: each computes fills_per_split fills into its own int32 partial sums
     int fills_per_split;
     int grid;
+    int px;                // 1: the layer suits the kernel that reads pre-expanded rows (lutgemm_px_kernel.hip)
 };
 
 // Quantization of one tensor as the pre-pass kernels see it.
@@ -101,6 +102,8 @@ struct DenseParams {
     const float *bias;           // not null: added to every output column after the epilogue
     int relu;                    // 1: max(x, 0) last
     int stagger_sleeps;          // s_sleep(127) periods by which every second group of workgroups starts late (0: none)
+    const uint16_t *px_rows;     // pre-expanded rows [n_col_tiles][fills / 2][256][128] (lutgemm_px_kernel only)
+    uint32_t px_bytes;
 };
 
 struct DepthwiseParams {
@@ -202,6 +205,10 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
 hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
                                 hipStream_t stream);
 hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream);
+// the same layer out of pre-expanded rows: launch_px_expand_rows builds p.px_rows from the packed filter codes
+hipError_t launch_px_expand_rows(const uint16_t *wq, const uint16_t *tableT, const DensePlan &plan, uint16_t *rows,
+                                 hipStream_t stream);
+hipError_t launch_dense_px(const DenseParams &p, bool out_i32, hipStream_t stream);
 hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials, float *out_f, int32_t *out_i,
                                   hipStream_t stream);
 hipError_t launch_axconv_correction(const uint8_t *codes, const uint8_t *fcodes, const ConvGeom &g, int offset_input,

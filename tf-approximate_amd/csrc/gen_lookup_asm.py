@@ -271,8 +271,135 @@ def emit(nt, buf):
             % (nt, buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))
 
 
+def emit_px(buf):
+    """PHASE_PX_B<buf>: one phase of the kernel variant that reads PRE-EXPANDED fills (16 columns per tile).
+
+    A fill here is a pair of ordinary fills: 8 input channels x 16 columns = 128 slots, so that the expanded row of
+    an activation code is 256 bytes, one pass over all 64 LDS banks.  The rows of a fill are built once per layer
+    in memory and a phase copies the next fill (64 KiB) straight into the other LDS buffer: eight buffer loads with
+    the lds modifier per wavefront, no transposition.  A lane owns two activation dwords per pixel and fill, FIRST
+    and SECOND; lanes with bit 3 set hold the two swapped, and read FIRST out of the upper half of the row, so that
+    the 16 lanes that share an LDS pass read 16 different 16-byte chunks.  A pixel is looked up as two units of
+    eight steps (FIRST, then SECOND) that run through the same rolling window of eight reads.
+
+    Buffer 1 lies 65536 bytes behind buffer 0, one more than the offset field of ds_read_b128 holds: its chunk
+    offsets carry 15 in their low four bits and the instruction adds 65521.
+    """
+    rows = 8
+    other = buf ^ 1
+
+    def read(st, r, h, step):
+        b = TEMP_BASE + 4 * step
+        va = ADDR_BASE + (step % 4)
+        st.ins("v_perm_b32 v%d, %%[%s%d], %%[ch%d%s], %%[s%d]" % (va, "fg"[h], r, h, "ab"[step >> 2], step))
+        off = " offset:65521" if buf else ""
+        return st.lds("ds_read_b128 v[%d:%d], v%d%s" % (b, b + 3, va, off))
+
+    def adds(st, r, steps):
+        g = steps[0] % 2
+        for d in range(4):
+            even = "%%[c%d_%d]" % (r, g * 8 + 2 * d)
+            odd = "%%[c%d_%d]" % (r, g * 8 + 2 * d + 1)
+            regs = [TEMP_BASE + 4 * step + d for step in steps]
+            st.ins("v_add3_u32 %s, %s, v%d, v%d" % (even, even, regs[0], regs[1]))
+            for reg in regs:
+                st.ins("v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
+                       % (odd, odd, reg))
+
+    groups = [(0, 2), (1, 3), (4, 6), (5, 7)]
+
+    def e_load(j):           # 1 KiB of the next fill: memory -> LDS buffer [other]
+        def f(st, state):
+            st.ins("s_add_u32 m0, %%[edst], %d" % (other * 65536 + j * 1024))
+            st.ins("s_add_u32 %%[stmp], %%[eoff], %d" % (j * 1024))
+            st.ins("buffer_load_dwordx4 %[l16], %[erc], %[stmp] offen lds")
+            st.ins("s_nop 0")
+        return f
+
+    def act_load(r):         # both activation dwords of pixel r for the next fill
+        def f(st, state):
+            st.ins("v_add_u32 v%d, %%[t%d], %%[dlf]" % (ADDR_BASE + 2, r))
+            st.ins("buffer_load_dword %%[nf%d], v%d, %%[xq], %%[qoff] offen" % (r, ADDR_BASE + 2))
+            st.ins("v_add_u32 v%d, %%[t%d], %%[dls]" % (ADDR_BASE + 3, r))
+            st.ins("buffer_load_dword %%[ng%d], v%d, %%[xq], %%[qoff] offen" % (r, ADDR_BASE + 3))
+        return f
+
+    aux = [e_load(j) for j in range(8)] + [act_load(r) for r in range(rows)]
+
+    def aux_step(st, state):
+        if state["pos"] < len(aux):
+            aux[state["pos"]](st, state)
+            state["pos"] += 1
+
+    def aux_rest(st, state):
+        while state["pos"] < len(aux):
+            aux_step(st, state)
+
+    def body(st, u, pending, with_next, state):
+        """Accumulate unit u = 2 * pixel + half; with_next: refill the window with unit u + 1."""
+        r, nxt = u // 2, [None] * 8
+        for steps in groups:
+            st.wait(max((pending[s] for s in steps), key=lambda op: st.fifo.index(op) if op in st.fifo else -1))
+            adds(st, r, steps)
+            for s in steps:
+                if with_next:
+                    nxt[s] = read(st, (u + 1) // 2, (u + 1) % 2, s)
+                aux_step(st, state)
+        return nxt
+
+    main = Stream()
+    main.ins("s_cmp_eq_u32 %[nr], 0")
+    main.ins("s_cbranch_scc1 Lzero_%=")
+    pending = [read(main, 0, 0, s) for s in range(8)]
+    state = {"pos": 0}
+    forks = []
+    for r in range(rows):
+        pending = body(main, 2 * r, pending, True, state)
+        if r < rows - 1:
+            main.ins("s_cmp_lt_u32 %d, %%[nr]" % (r + 1))
+            main.ins("s_cbranch_scc0 Llast%d_%%=" % r)
+            forks.append((r, main.fork(), list(pending), dict(state)))
+            pending = body(main, 2 * r + 1, pending, True, state)
+        else:
+            body(main, 2 * r + 1, pending, False, state)
+    aux_rest(main, state)
+    main.drain()
+    main.ins("s_branch Lend_%=")
+    for r, st, pend, stt in forks:
+        st.label("Llast%d_%%=" % r)
+        body(st, 2 * r + 1, pend, False, stt)
+        aux_rest(st, stt)
+        st.drain()
+        st.ins("s_branch Lend_%=")
+    zero = Stream(main.lines)
+    zero.label("Lzero_%=")
+    aux_rest(zero, {"pos": 0})
+    zero.drain()
+    zero.label("Lend_%=")
+
+    outs = ['[c%d_%d] "+v"(ACC[%d][%d])' % (r, i, r, i) for r in range(rows) for i in range(16)]
+    outs += ['[nf%d] "=&v"(NFIRST[%d])' % (r, r) for r in range(rows)]
+    outs += ['[ng%d] "=&v"(NSECOND[%d])' % (r, r) for r in range(rows)]
+    outs += ['[stmp] "=&s"(STMP)']
+    inp = ['[f%d] "v"(FIRST[%d])' % (r, r) for r in range(rows)]
+    inp += ['[g%d] "v"(SECOND[%d])' % (r, r) for r in range(rows)]
+    inp += ['[t%d] "v"(TAPOFF[%d])' % (r, r) for r in range(rows)]
+    inp += ['[s%d] "v"(SEL[%d])' % (i, i) for i in range(8)]
+    inp += ['[ch0a] "v"(CH[0])', '[ch0b] "v"(CH[1])', '[ch1a] "v"(CH[2])', '[ch1b] "v"(CH[3])']
+    inp += ['[dlf] "v"(DLF)', '[dls] "v"(DLS)', '[l16] "v"(L16)', '[nr] "s"(NR)']
+    inp += ['[edst] "s"(EDST)', '[eoff] "s"(EOFF)', '[erc] "s"(ERC)', '[xq] "s"(XQ)', '[qoff] "s"(QOFF)']
+    clob = ", ".join('"v%d"' % r for r in range(ADDR_BASE, TEMP_BASE + 32))
+    body_text = " \\\n        ".join(main.lines)
+    args = "ACC, FIRST, SECOND, NFIRST, NSECOND, TAPOFF, SEL, CH, DLF, DLS, L16, NR, STMP, EDST, EOFF, ERC, XQ, QOFF"
+    return ("#define PHASE_PX_B%d(%s) \\\n    asm volatile( \\\n        %s \\\n"
+            "        : %s \\\n        : %s \\\n        : %s, \"scc\", \"memory\")\n"
+            % (buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))
+
+
 if __name__ == "__main__":
     print("// Generated by gen_lookup_asm.py -- do not edit.")
     for nt in (16, 32, 64):
         for buf in (0, 1):
             print(emit(nt, buf))
+    for buf in (0, 1):
+        print(emit_px(buf))

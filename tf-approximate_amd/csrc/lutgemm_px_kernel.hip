@@ -1,0 +1,255 @@
+// Dense LUT-GEMM out of PRE-EXPANDED rows (gfx950), for layers with many output pixels and a small filter.
+//
+// lutgemm_kernel.hip builds the expanded rows of every fill inside every workgroup: table rows are staged in LDS
+// and transposed, once per (tile, fill).  Here px_expand_rows_kernel builds them once per layer in memory:
+//
+//   E[column tile][fill][phys_row(a)][slot]  = T[a][filter code of slot],   256 rows x 128 slots x uint16 = 64 KiB
+//
+// where a fill is a PAIR of the other kernel's fills: 8 input channels (two channel quads of one tap) x 16 columns,
+// slot = quad-in-pair * 64 + channel-in-quad * 16 + column.  The lookup kernel then only copies fills from memory
+// (L2: the workgroups of an XCD walk the same few column tiles at the same time) straight into LDS with buffer
+// loads that carry the lds modifier - no staged table rows, no transposition, half as many barriers - and, because
+// an expanded row is now 256 bytes, a 64-lane ds_read_b128 spreads over all 64 banks.
+//
+// LDS: two fill buffers of 64 KiB, then the parked pixel geometry (32 KiB).  While fill p is looked up out of one
+// buffer, fill p + 1 lands in the other; a tile starts in buffer 0, which receives the first fill of the
+// workgroup's next tile as soon as the last fill that used it is done, and the epilogue turns its outputs through
+// buffer 1.
+//
+// Restates ApproxConvIm2ColKernel + ApproxConvGEMMKernel (tf2/src/approx_nn_conv_kernels.cpp:215-296) like the
+// other kernel; results are bit-identical to it (same int32 sums, same epilogue).
+#include "lutgemm_tile.h"
+#include "lookup_asm.inc"
+
+namespace axc {
+
+extern __shared__ __align__(16) unsigned char lds_px[];
+
+constexpr int kPxFillBytes = 65536;     // one pre-expanded fill: 256 activation rows x 128 slots x uint16
+constexpr int kPxBlockCols = 4;         // column tiles that the workgroups of an XCD walk side by side
+
+// One workgroup per quarter of a (column tile, fill): thread a gathers 32 of the 128 entries of activation code a
+// (32 independent two-byte loads out of the L2-resident table, coalesced over a) and stores them as 64 bytes.
+__global__ void __launch_bounds__(256) px_expand_rows_kernel(const uint16_t *__restrict__ wq,
+                                                             const uint16_t *__restrict__ tableT, const int fills,
+                                                             uint16_t *__restrict__ rows)
+{
+    const int px_fills = fills / 2;
+    const int block = (int)blockIdx.x >> 2, quarter = (int)blockIdx.x & 3;
+    const int ct = block / px_fills, f = block - ct * px_fills;
+    // the codes of the two ordinary fills of this pair lie side by side: 128 uint16
+    const uint16_t *codes = wq + ((size_t)ct * fills + 2 * (size_t)f) * 64 + quarter * 32;
+    const uint32_t a = threadIdx.x;
+    typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+    u32x4s *dst = reinterpret_cast<u32x4s *>(rows + (size_t)block * (kPxFillBytes / 2) + phys_row(a) * 128u + quarter * 32);
+    uint32_t w[16];
+#pragma unroll
+    for (int d = 0; d < 16; ++d) {
+        const uint32_t lo = tableT[(uint32_t)codes[2 * d] * 256u + a];
+        const uint32_t hi = tableT[(uint32_t)codes[2 * d + 1] * 256u + a];
+        w[d] = lo | (hi << 16);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        u32x4s v = {w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]};
+        dst[k] = v;
+    }
+}
+
+hipError_t launch_px_expand_rows(const uint16_t *wq, const uint16_t *tableT, const DensePlan &plan, uint16_t *rows,
+                                 hipStream_t stream)
+{
+    const int blocks = plan.n_col_tiles * (plan.fills / 2) * 4;
+    hipLaunchKernelGGL(px_expand_rows_kernel, dim3(blocks), dim3(256), 0, stream, wq, tableT, plan.fills, rows);
+    return hipGetLastError();
+}
+
+template <bool OUT_I32>
+__global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DenseParams p)
+{
+    constexpr int NT = 16, R = 8;
+    const ConvGeom &g = p.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // ---- lane constants ----
+    // A pixel is looked up in two units of eight steps, one per activation dword.  Step s of a unit reads chunk
+    // (c0 + s) & 7 of one half of the 256-byte row; lanes with bit 3 set keep their two dwords swapped and read the
+    // upper half first, so the 16 lanes of an LDS pass touch 16 different chunks whatever their codes are.
+    // Chunk c of a half holds input channel c >> 1 of its quad, column group c & 1.  The address
+    // (row << 8 | half << 7 | c << 4) is one v_perm_b32: byte 1 <- activation byte c >> 1, byte 0 <- the chunk byte.
+    const int c0 = lane & 7;
+    const uint32_t upper = ((uint32_t)lane >> 3) & 1u;
+    uint32_t sel[8];
+    uint32_t ch[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};   // [buffer][unit * 2 + (step >> 2)]: four chunk bytes each
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const uint32_t c = (uint32_t)(c0 + s) & 7u;
+        sel[s] = 0x0c0c0000u | ((4u + (c >> 1)) << 8) | (uint32_t)(s & 3);
+#pragma unroll
+        for (int unit = 0; unit < 2; ++unit) {
+            const uint32_t half = (uint32_t)unit ^ upper;
+            const uint32_t byte = ((half << 3) | c) << 4;
+            ch[0][unit * 2 + (s >> 2)] |= byte << (8 * (s & 3));
+            // buffer 1 starts 65536 bytes in, one more than an instruction offset holds: +15 here, +65521 there
+            ch[1][unit * 2 + (s >> 2)] |= (byte | 15u) << (8 * (s & 3));
+        }
+    }
+    const uint32_t l16 = (uint32_t)lane * 16u;
+    uint32_t *const park = reinterpret_cast<uint32_t *>(lds_px + 2 * kPxFillBytes) + tid;
+
+    const int n_col = p.plan.n_col_tiles, n_row = p.plan.n_row_tiles;
+    const int ntiles = n_row * n_col;
+    const int F = p.plan.fills / 2;                 // pre-expanded fills over K
+    const int qpairs = g.C4 / 2;                    // fills per tap
+    const uint32_t quad_bytes = (uint32_t)g.W * 4u; // between the channel quads of a pixel in xq
+    const uint32_t dlf = upper ? quad_bytes : 0u;   // this lane's FIRST dword is the pair's second quad if swapped
+    const uint32_t dls = upper ? 0u : quad_bytes;
+    const uint32_t zp_row = p.xq_bytes;             // one extra input row of the zero-point code behind xq
+    const rsrc_t xq_rsrc = make_rsrc(p.xq, p.xq_bytes + (uint32_t)(g.C4 * g.W) * 4u);
+    const rsrc_t e_rsrc = make_rsrc(p.px_rows, p.px_bytes);
+
+    // Tiles in blocks of kPxBlockCols column tiles: inside a block row tile after row tile, the column tile fastest.
+    // Workgroups with neighbouring indices sit on one XCD (own L2) and work on neighbouring tiles: the same few
+    // column tiles (same pre-expanded rows) of a few row tiles (same activations).
+    auto decode = [&](const int tile, int &rt, int &ct) __attribute__((always_inline)) {
+        const int per_block = n_row * kPxBlockCols;
+        const int cb = tile / per_block;
+        const int in_block = tile - cb * per_block;
+        const int left = n_col - cb * kPxBlockCols;
+        const int w = left < kPxBlockCols ? left : kPxBlockCols;
+        rt = in_block / w;
+        ct = cb * kPxBlockCols + in_block - rt * w;
+    };
+    const int G = (int)gridDim.x;
+    const int wg = (G & 7) == 0 ? ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
+    if (p.stagger_sleeps && ((wg / (n_col < kPxBlockCols ? n_col : kPxBlockCols)) & 1))
+        for (int i = 0; i < p.stagger_sleeps; ++i)
+            __builtin_amdgcn_s_sleep(127);
+
+    int prev_rt = -1;
+    uint32_t nr = 0;
+    const uint32_t edst = (uint32_t)wave * 8192u;   // this wavefront's eighth of a fill, in memory and in LDS
+    // fill 0 of a column tile -> buffer 0: eight loads of 1 KiB, memory straight into LDS
+    auto load_first_fill = [&](const int ct) __attribute__((always_inline)) {
+        const uint32_t eoff = (uint32_t)(ct * F) * (uint32_t)kPxFillBytes + edst;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                e_rsrc, (__attribute__((address_space(3))) void *)(lds_px + edst + j * 1024u), 16, (int)l16,
+                (int)(eoff + j * 1024u), 0, 0);
+    };
+    if (wg < ntiles) {
+        int rt0, ct0;
+        decode(wg, rt0, ct0);
+        load_first_fill(ct0);
+    }
+    for (int tile = wg; tile < ntiles; tile += G) {
+        int rt, ct;
+        decode(tile, rt, ct);
+        int ct_next = ct;
+        const bool has_next = tile + G < ntiles;
+        if (has_next) {
+            int rt_next;
+            decode(tile + G, rt_next, ct_next);
+        }
+        const TileRows t = tile_rows_of<R>(p, rt, wave);
+        if (rt != prev_rt) {
+            prev_rt = rt;
+            nr = park_geometry<R>(p, t, lane, park);
+        }
+        const uint32_t nr_s = __builtin_amdgcn_readfirstlane(nr);
+
+        // ---- activation cursor: (tap, quad pair) of the fill whose activations are fetched next ----
+        int cur_fill = 0, cur_qp = 0, cur_kh = 0, cur_kw = 0;
+        uint32_t idx_tap[R];
+        tap_offsets<R>(g, park, 0, 0, zp_row, idx_tap);
+        auto advance_cursor = [&]() __attribute__((always_inline)) {
+            ++cur_fill;
+            if (++cur_qp == qpairs) {
+                cur_qp = 0;
+                if (++cur_kw == g.KW) { cur_kw = 0; ++cur_kh; }
+                if (cur_fill < F)
+                    tap_offsets<R>(g, park, cur_kh, cur_kw, zp_row, idx_tap);
+            }
+        };
+        uint32_t fA[R], sA[R], fB[R], sB[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            fA[r] = ld_u32(xq_rsrc, idx_tap[r] + dlf, 0);
+            sA[r] = ld_u32(xq_rsrc, idx_tap[r] + dls, 0);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of fill 0 and its activations are there
+        __syncthreads();                      // ... and everyone's; the previous tile's epilogue is done with LDS
+
+        int32_t acc[R][NT];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+                acc[r][j] = 0;
+
+        if (F > 1)
+            advance_cursor();   // entering phase p the cursor stands on fill p + 1
+        auto phase = [&](const int pcur, uint32_t (&f_cur)[R], uint32_t (&s_cur)[R], uint32_t (&f_next)[R],
+                         uint32_t (&s_next)[R], auto buf_tag) __attribute__((always_inline)) {
+            constexpr int BUF = decltype(buf_tag)::value;
+            // What lands in the other buffer during this phase: the next fill of this tile.  Behind the last fill of
+            // an even count the other buffer is buffer 0, and it gets the first fill of the workgroup's next tile;
+            // otherwise the last fill once more (never used).
+            uint32_t fill_next = (uint32_t)(ct * F + pcur + 1);
+            if (pcur + 1 >= F)
+                fill_next = (BUF == 1 && has_next) ? (uint32_t)(ct_next * F) : (uint32_t)(ct * F + F - 1);
+            const uint32_t eoff = fill_next * (uint32_t)kPxFillBytes + edst;
+            const uint32_t qoff = (uint32_t)cur_qp * 2u * quad_bytes;
+            uint32_t stmp;
+            if constexpr (BUF == 0)
+                PHASE_PX_B0(acc, f_cur, s_cur, f_next, s_next, idx_tap, sel, ch[0], dlf, dls, l16, nr_s, stmp,
+                            __builtin_amdgcn_readfirstlane(edst), __builtin_amdgcn_readfirstlane(eoff), e_rsrc, xq_rsrc,
+                            __builtin_amdgcn_readfirstlane(qoff));
+            else
+                PHASE_PX_B1(acc, f_cur, s_cur, f_next, s_next, idx_tap, sel, ch[1], dlf, dls, l16, nr_s, stmp,
+                            __builtin_amdgcn_readfirstlane(edst), __builtin_amdgcn_readfirstlane(eoff), e_rsrc, xq_rsrc,
+                            __builtin_amdgcn_readfirstlane(qoff));
+            (void)stmp;
+            if (pcur + 2 < F)
+                advance_cursor();
+            __syncthreads();
+        };
+        for (int pcur = 0; pcur < F; pcur += 2) {
+            phase(pcur, fA, sA, fB, sB, std::integral_constant<int, 0>());
+            if (pcur + 1 < F)
+                phase(pcur + 1, fB, sB, fA, sA, std::integral_constant<int, 1>());
+        }
+        // An odd count of fills ends on buffer 0, which every wavefront has now left: the next tile's first fill
+        // goes there while the epilogue runs.  The epilogue turns its outputs through buffer 1 either way.
+        if ((F & 1) && has_next)
+            load_first_fill(ct_next);
+        fix_even_columns<R, NT>(acc);
+        store_tile<NT, OUT_I32>(p, acc, t, ct, 0, nr_s, lane, wave, lds_px + kPxFillBytes);
+    }
+}
+
+template <bool OUT_I32>
+static hipError_t launch_px_one(const DenseParams &p, hipStream_t stream)
+{
+    auto kernel = lutgemm_px_kernel<OUT_I32>;
+    // The generated assembly addresses LDS from offset 0: that holds as long as the kernel has no static LDS in
+    // front of its dynamic allocation (checked when the attribute is set, once per device).
+    const int lds_bytes = 2 * kPxFillBytes + kDenseParkBytes;
+    const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(kernel), lds_bytes, true);
+    if (e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kernel, dim3(p.plan.grid), dim3(kDenseThreads), lds_bytes, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_px(const DenseParams &p, bool out_i32, hipStream_t stream)
+{
+    if (p.plan.nt != 16 || p.plan.k_splits != 1 || (p.plan.fills & 1) || (p.g.C4 & 1) || !p.px_rows)
+        return hipErrorInvalidValue;
+    return out_i32 ? launch_px_one<true>(p, stream) : launch_px_one<false>(p, stream);
+}
+
+} // namespace axc

@@ -334,6 +334,11 @@ def set_tile_columns(columns):
     _check(_lib.load().axc_set_tile_columns(int(columns)))
 
 
+def set_preexpand(mode):
+    """Which dense layers run out of pre-expanded rows: 0 = the planner's choice, 1 = all that can, -1 = none."""
+    _check(_lib.load().axc_set_preexpand(int(mode)))
+
+
 _table_cache = {}
 
 
