@@ -22,10 +22,8 @@
 //
 // Restates, as one fused kernel, what the reference does in ApproxConvIm2ColKernel +
 // ApproxConvGEMMKernel (tf2/src/approx_nn_conv_kernels.cpp:215-296) per chunk.
-#include "axconv_internal.h"
+#include "lutgemm_tile.h"
 #include "lookup_asm.inc"
-
-#include <type_traits>
 
 namespace axc {
 
@@ -33,24 +31,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 extern __shared__ __align__(16) unsigned char lds[];
-
-// Global loads go through raw buffer descriptors: address = SGPR base + SGPR offset + one 32-bit VGPR
-// offset, so no load needs a 64-bit VGPR address, and reads past the end return 0 instead of faulting.
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ uint32_t ld_u32(rsrc_t r, uint32_t voff, uint32_t soff)
-{
-    return __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
-}
-__device__ __forceinline__ u32x2 ld_u32x2(rsrc_t r, uint32_t voff, uint32_t soff)
-{
-    return __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0);
-}
-
-constexpr int kOldShare = 11; // sixteenths of a tile's wavefront-rows owned by the older four wavefronts
 
 template <int NT>
 struct DenseCfg {
@@ -162,7 +142,6 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         for (int i = 0; i < p.stagger_sleeps; ++i)
             __builtin_amdgcn_s_sleep(127);
     int prev_rt = -1;
-    bool rvalid[DenseCfg<NT>::R];    // this lane's pixel exists
     uint32_t nr = 0;                 // pixels of this lane whose wavefront row exists (a prefix; wave-uniform)
     for (int tile = wg; tile < ntiles; tile += G) {
         const int rt = tile / nct_v;
@@ -171,63 +150,13 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         ct -= ksi * p.plan.n_col_tiles;
         const int f0 = ksi * p.plan.fills_per_split;        // its fills: [f0, f0 + fills)
         const int fills = fills_all - f0 < p.plan.fills_per_split ? fills_all - f0 : p.plan.fills_per_split;
-        const int64_t row0 = (int64_t)rt * p.plan.rows_per_tile;
-        const int64_t row_end = (row0 + p.plan.rows_per_tile < g.M) ? row0 + p.plan.rows_per_tile : g.M;
-
-        // ---- which wavefront-rows (64 consecutive output pixels) of the tile this wavefront owns ----
-        // The SIMD issues the older of its two wavefronts first, so the first four wavefronts get through
-        // their lookups faster; they own kOldShare/16 of the tile, and both halves reach the barrier together.
-        const int wrows = (int)((row_end - row0 + 63) / 64);
-        int wr_old = (wrows * kOldShare + 8) / 16;
-        wr_old = wr_old > 4 * R ? 4 * R : wr_old;
-        wr_old = wr_old < wrows - 4 * R ? wrows - 4 * R : wr_old;
-        const bool old_half = wave < kDenseWaves / 2;
-        const int wr_base = old_half ? wave : wr_old + wave - kDenseWaves / 2; // then every fourth wavefront-row
-        const int64_t wr_end = row0 + (int64_t)(old_half ? wr_old : wrows) * 64;
-
-        // ---- per-pixel geometry (parked in LDS, in slots private to the thread; only read back when the tap
-        // changes).  It depends on the row tile alone: kept from the previous tile when that had the same one.
+        // ---- which wavefront-rows (64 consecutive output pixels) of the tile this wavefront owns, and the
+        // per-pixel geometry (parked in LDS, in slots private to the thread; only read back when the tap changes).
+        // The geometry depends on the row tile alone: kept from the previous tile when that had the same one.
+        const TileRows t = tile_rows_of<R>(p, rt, wave);
         if (rt != prev_rt) {
             prev_rt = rt;
-            nr = 0;
-            // (n, oh, ow) of this lane's first pixel by division; its further pixels lie a fixed number of output
-            // pixels apart (four wavefront-rows), so they follow by adding that step's (n, oh, ow) with carries
-            int n = 0, oh = 0, ow = 0;
-            {
-                const int64_t m0 = row0 + (int64_t)wr_base * 64 + lane;
-                const int64_t mm = m0 < g.M ? m0 : 0;
-                int rem;
-                if (g.M <= 0x7fffffff) { // the usual case: 32-bit divisions (a 64-bit one costs several times more)
-                    const uint32_t ohow = (uint32_t)(g.OH * g.OW);
-                    n = (int)((uint32_t)mm / ohow);
-                    rem = (int)((uint32_t)mm - (uint32_t)n * ohow);
-                } else {
-                    n = (int)(mm / ((int64_t)g.OH * g.OW));
-                    rem = (int)(mm - (int64_t)n * g.OH * g.OW);
-                }
-                oh = (int)((uint32_t)rem / (uint32_t)g.OW);
-                ow = rem - oh * g.OW;
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int64_t wrow = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
-                nr += (wrow < row_end && wrow < wr_end) ? 1u : 0u;
-                const int64_t m = wrow + lane;
-                rvalid[r] = m < row_end && wrow < wr_end;
-                const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
-                // dword index in xq of tap (0, 0), channel quad 0 (may point outside the image)
-                park[(2 * r) * kDenseThreads] = rvalid[r] ? (uint32_t)((n * g.H + ih0) * rowstep + iw0) : 0u;
-                // input coordinates of tap (0, 0); ih0 = -32768 marks a pixel that does not exist
-                park[(2 * r + 1) * kDenseThreads] = rvalid[r] ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
-                // the next pixel of this lane: p.step_* = (n, oh, ow) of 64 * kDenseWaves / 2 output pixels
-                ow += p.step_ow;
-                const int c1 = ow >= g.OW ? 1 : 0;
-                ow -= c1 ? g.OW : 0;
-                oh += p.step_oh + c1;
-                const int c2 = oh >= g.OH ? 1 : 0;
-                oh -= c2 ? g.OH : 0;
-                n += p.step_n + c2;
-            }
+            nr = park_geometry<R>(p, t, lane, park);
         }
 
         const uint32_t wq_tile = ((uint32_t)ct * (uint32_t)fills_all + (uint32_t)f0) * 128u; // this tile's first codes
@@ -237,19 +166,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         int cur_fill = 0, cur_sub = f0 % SUBS;
         int cur_q = (f0 / SUBS) % g.C4, cur_kh = (f0 / SUBS / g.C4) / g.KW, cur_kw = (f0 / SUBS / g.C4) % g.KW;
         uint32_t idx_tap[R];   // byte offset in xq of quad 0 of the current tap (the zero-point row outside)
-        auto tap_setup = [&]() {
-            const int dh = cur_kh * g.dh, dw = cur_kw * g.dw;
-            const int tap_off = dh * rowstep + dw;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int32_t pb = (int32_t)park[(2 * r) * kDenseThreads];
-                const int32_t hw = (int32_t)park[(2 * r + 1) * kDenseThreads];
-                const int ih = (hw >> 16) + dh;
-                const int iw = (int)(int16_t)(hw & 0xffff) + dw;
-                const bool inb = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-                idx_tap[r] = inb ? (uint32_t)((pb + tap_off) * 4) : zp_row;
-            }
-        };
+        auto tap_setup = [&]() { tap_offsets<R>(g, park, cur_kh, cur_kw, zp_row, idx_tap); };
         auto load_acts = [&](uint32_t (&dst)[R]) {
             const uint32_t qoff = (uint32_t)(cur_q * g.W * 4); // scalar: channel quad inside the pixel row
 #pragma unroll
@@ -379,170 +296,9 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
                 phase(pcur + 1, actB, actA, std::integral_constant<int, 1>());
         }
 
-        // The phases add whole dwords (two 16-bit table entries) into the accumulator of the even column and the
-        // high entry alone into that of the odd column: even = sum(lo) + 65536 * sum(hi) modulo 2^32.
-        // Subtracting a multiple of 65536 changes the high half only: one 16-bit subtract (high half of the even
-        // accumulator minus low half of the odd one, written back into the high half, low half kept).
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int j = 0; j < NT; j += 2)
-                __asm__("v_sub_u16_sdwa %0, %0, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1 src1_sel:WORD_0"
-                        : "+v"(acc[r][j])
-                        : "v"(acc[r][j + 1]));
-
-        // ---- epilogue: zero-point correction + dequantize (approx_nn_conv_kernels.cpp:250-253) ----
-        // A lane holds NT consecutive columns of its pixel: stored as they are, one instruction would touch 64
-        // different 64-byte pieces of memory.  The wavefront therefore turns each of its wavefront-rows
-        // through a private piece of LDS (every buffer is free after the last phase) so that NT/4 neighbouring
-        // lanes write one pixel's NT columns: 16 or 8 contiguous runs per store instruction.
-        const float e_s1xs2 = p.lq_dev ? p.lq_dev->s1xs2 : p.s1xs2, e_m1 = p.lq_dev ? p.lq_dev->m1 : p.m1;
-        const float e_m2 = p.lq_dev ? p.lq_dev->m2 : p.m2, e_km = p.lq_dev ? p.lq_dev->k_m1xm2 : p.k_m1xm2;
-        // what the Keras layer does behind the op (bias_add, then the activation): fused into the store
-        auto finish = [&](float v, int col) {
-            if (p.bias)
-                v = __fadd_rn(v, p.bias[col]);
-            return p.relu ? fmaxf(v, 0.0f) : v;
-        };
-        constexpr bool kTransposed = NT <= 32;
-        // Every global load of the epilogue is issued here, ahead of the first store: loads and stores complete in
-        // issue order, so a load behind a store would wait until that store has reached memory.
-        float ps[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int64_t m = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64 + lane;
-            ps[r] = (!OUT_I32 && rvalid[r]) ? p.psum[m] : 0.0f;
-        }
-        if (kTransposed && (g.Co & 3) == 0) {
-            constexpr int Q = NT / 4;                 // 16-byte quads (lanes) per pixel
-            constexpr int PITCH = NT * 4 + 16;        // bytes per pixel in LDS: the +16 spreads pixels over the banks
-            unsigned char *const wl = lds + (size_t)wave * 64 * PITCH;
-            typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
-            // Behind the transposition a lane stores the same four columns of every pixel it handles: the terms
-            // that depend on the column (filter sum, bias) are applied there, from four registers each.
-            const int quad = lane % Q, colq = ct * NT + quad * 4;
-            float t3q[4], biasq[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int c = colq + j < g.Co ? colq + j : g.Co - 1;
-                t3q[j] = OUT_I32 ? 0.0f : __fmul_rn(e_m1, p.fsum[c]);
-                biasq[j] = (!OUT_I32 && p.bias) ? p.bias[c] : 0.0f;
-            }
-            // bias and ReLU are wave-uniform run-time switches: one copy of the store loop per combination, chosen
-            // once, instead of two selects per output element
-            auto store_rows = [&](auto has_bias_t, auto has_relu_t) {
-            constexpr bool kBias = decltype(has_bias_t)::value, kRelu = decltype(has_relu_t)::value;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (r >= (int)nr_s)
-                    break;
-                const int64_t m0 = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64;
-                const int nvalid = (int)(row_end - m0 < 64 ? row_end - m0 : 64);
-                const float t1 = __fmul_rn(e_m2, ps[r]);
-#pragma unroll
-                for (int set = 0; set < SETS; ++set) {
-                    const int h = (c0 + set) & (SETS - 1);
-                    uint32_t w[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        if (OUT_I32)
-                            w[e] = (uint32_t)acc[r][set * 8 + e];
-                        else
-                            w[e] = __float_as_uint(__fadd_rn(__fmul_rn((float)acc[r][set * 8 + e], e_s1xs2), t1));
-                    }
-                    u32x4s lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
-                    *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32) = lo;
-                    *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32 + 16) = hi;
-                }
-                uint32_t *const out = OUT_I32 ? reinterpret_cast<uint32_t *>(p.out_i) + (int64_t)ksi * g.M * g.Co
-                                              : reinterpret_cast<uint32_t *>(p.out_f);
-#pragma unroll
-                for (int i = 0; i < Q; ++i) {
-                    const int pix = i * (64 / Q) + lane / Q;
-                    u32x4s d = *reinterpret_cast<const u32x4s *>(wl + pix * PITCH + quad * 16);
-                    if (!OUT_I32) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            float v = __fsub_rn(__fadd_rn(__uint_as_float(d[j]), t3q[j]), e_km);
-                            if (kBias)
-                                v = __fadd_rn(v, biasq[j]);
-                            d[j] = __float_as_uint(kRelu ? fmaxf(v, 0.0f) : v);
-                        }
-                    }
-                    if (pix < nvalid && colq < g.Co) {
-                        // the float output is not read again by this op: streamed past the caches, which keeps
-                        // them for the activations; split-K partial sums are read back at once and stay cached
-                        if (OUT_I32)
-                            *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq) = d;
-                        else
-                            __builtin_nontemporal_store(d, reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq));
-                    }
-                }
-            }
-            };
-            using yes = std::true_type;
-            using no = std::false_type;
-            if (OUT_I32 || (!p.bias && !p.relu))
-                store_rows(no(), no());
-            else if (p.bias && p.relu)
-                store_rows(yes(), yes());
-            else if (p.bias)
-                store_rows(yes(), no());
-            else
-                store_rows(no(), yes());
-            continue;
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if (!rvalid[r])
-                continue;
-            const int64_t m = row0 + (int64_t)(wr_base + r * (kDenseWaves / 2)) * 64 + lane;
-            // patch sum of the raw input in the reference's order (tap-major, channels ascending)
-            const float t1 = __fmul_rn(e_m2, ps[r]);
-#pragma unroll
-            for (int set = 0; set < SETS; ++set) {
-                const int h = (c0 + set) & (SETS - 1);
-                const int col0 = ct * NT + h * 8;
-                if (col0 >= g.Co)
-                    continue;
-                const int64_t o = m * g.Co + col0;
-                const bool vec = (g.Co & 3) == 0 && col0 + 8 <= g.Co; // 32 contiguous, 16-byte aligned bytes
-                if (OUT_I32) {
-                    if (vec) {
-                        typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-                        i32x4 lo = {acc[r][set * 8 + 0], acc[r][set * 8 + 1], acc[r][set * 8 + 2], acc[r][set * 8 + 3]};
-                        i32x4 hi = {acc[r][set * 8 + 4], acc[r][set * 8 + 5], acc[r][set * 8 + 6], acc[r][set * 8 + 7]};
-                        *reinterpret_cast<i32x4 *>(p.out_i + (int64_t)ksi * g.M * g.Co + o) = lo;
-                        *reinterpret_cast<i32x4 *>(p.out_i + (int64_t)ksi * g.M * g.Co + o + 4) = hi;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (col0 + e < g.Co)
-                                p.out_i[(int64_t)ksi * g.M * g.Co + o + e] = acc[r][set * 8 + e];
-                    }
-                } else {
-                    float v[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int col = col0 + e < g.Co ? col0 + e : g.Co - 1;
-                        const float t0 = __fmul_rn((float)acc[r][set * 8 + e], e_s1xs2);
-                        const float t2 = __fadd_rn(t0, t1);
-                        const float t3 = __fmul_rn(e_m1, p.fsum[col]);
-                        const float t4 = __fadd_rn(t2, t3);
-                        v[e] = finish(__fsub_rn(t4, e_km), col);
-                    }
-                    if (vec) {
-                        *reinterpret_cast<float4 *>(p.out_f + o) = make_float4(v[0], v[1], v[2], v[3]);
-                        *reinterpret_cast<float4 *>(p.out_f + o + 4) = make_float4(v[4], v[5], v[6], v[7]);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (col0 + e < g.Co)
-                                p.out_f[o + e] = v[e];
-                    }
-                }
-            }
-        }
+        fix_even_columns<R, NT>(acc);
+        // every buffer is free after the last phase: the epilogue turns its outputs through the expanded rows
+        store_tile<NT, OUT_I32>(p, acc, t, ct, ksi, nr_s, lane, wave, lds);
     }
 }
 
