@@ -419,14 +419,14 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
         }
     }
     // Pre-expanded rows: 16-column tiles over the whole K, channel quads in pairs.  They cost 512 bytes of memory per
-    // filter element, written once per call (one more launch: ~7 us, then ~3 TB/s) and read once per XCD; the lookup
-    // kernel then runs about an eighth faster (measured: 11-14 % at ~24 T lookups/s).  Worth it with many output
+    // filter element, written once per call (one more launch: ~6.5 us, then ~5 TB/s) and read once per XCD; the lookup
+    // kernel then runs about an eighth faster (measured: 10-15 % at ~24 T lookups/s).  Worth it with many output
     // pixels per filter element.
     best.px = 0;
     const size_t px_bytes = (size_t)best.n_col_tiles * (size_t)(best.fills / 2) * 65536;
     if (px_mode >= 0 && best.nt == 16 && best.k_splits == 1 && (g.C4 & 1) == 0 && px_bytes <= kPxMaxBytes) {
         const double lookups = (double)g.M * (double)best.fills * 4.0 * (double)best.n_col_tiles * 16.0;
-        const double gain_s = 0.11 * lookups / 24e12, cost_s = 7e-6 + (double)px_bytes / 3e12;
+        const double gain_s = 0.12 * lookups / 24e12, cost_s = 6.5e-6 + (double)px_bytes / 5e12;
         best.px = (px_mode > 0 || gain_s > cost_s) ? 1 : 0;
     }
     return best;
