@@ -71,24 +71,29 @@ LAYERS = [
     ("cfg5_stress", "B_3x3_512_512", (64, 28, 28, 512), (3, 3, 512, 512), (1, 1), False, "halfnormal", "random"),
 ]
 
-# HBM bytes per launch of the main kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each
-# scaled by what the same counter reads for --copy-calibration.  Not measured in the run that prints them: the
-# bench line says which profile they come from.
+# Bytes per launch that the main kernel moves between its L2s and the memory side (Infinity Cache or HBM), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for the
+# device copy of known size inside the same run.  Keyed by (workload, kernel); not measured in the run that prints
+# them: the bench line says which profile they come from.
 PROFILED_TRAFFIC = {
-    "conv3x3_b64_56x56x64_to_64_s1_same": (2.000 * 8034.0 * 1024 + 1.000 * 61573.5 * 1024,
-                                           "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
-    "conv1x1_b64_112x112x32_to_192": (2.000 * 19020.5 * 1024 + 1.000 * 731723.0 * 1024,
-                                      "profiles/lutgemm_expand_conv1x1_b64_112x112x32_to_192.md"),
-    "conv1x1_b64_56x56x64_to_256": (2.000 * 8133.0 * 1024 + 1.000 * 253711.0 * 1024,
-                                    "profiles/lutgemm_expand_conv1x1_b64_56x56x64_to_256.md"),
-    "conv7x7s2_b64_224x224x3_to_64": (2.000 * 9278.5 * 1024 + 1.000 * 231414.8 * 1024,
-                                      "profiles/lutgemm_expand_conv7x7s2_b64_224x224x3_to_64.md"),
-    "conv1x1_b32_56x56x256_to_1024": (2.000 * 27862.1 * 1024 + 1.000 * 486248.0 * 1024,
-                                      "profiles/lutgemm_expand_conv1x1_b32_56x56x256_to_1024.md"),
-    "dw3x3_b64_112x112x192_s1": (2.000 * 342889 * 1024 + 1.000 * 602112 * 1024,
-                                 "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
-    "dw3x3_b64_112x112x192_s2": (2.000 * 321245 * 1024 + 1.000 * 150528 * 1024,
-                                 "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 80798.1 * 1024 + 1.000 * 59255.0 * 1024,
+                                                           "profiles/lutgemm_px_conv3x3_b64_56x56x64.md"),
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8293.5 * 1024 + 1.000 * 61660.2 * 1024,
+                                                               "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
+    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 55035.8 * 1024 + 1.000 * 800538.5 * 1024,
+                                                      "profiles/lutgemm_px_conv1x1_b64_112x112x32_to_192.md"),
+    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 46293.2 * 1024 + 1.000 * 270570.7 * 1024,
+                                                    "profiles/lutgemm_px_conv1x1_b64_56x56x64_to_256.md"),
+    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 466574.7 * 1024 + 1.000 * 484717.4 * 1024,
+                                                      "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
+    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_expand"): (2.000 * 9530.0 * 1024 + 1.000 * 245053.4 * 1024,
+                                                          "profiles/lutgemm_expand_conv7x7s2_b64_224x224x3_to_64.md"),
+    ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51685.6 * 1024 + 1.000 * 106840.3 * 1024,
+                                                         "profiles/lutgemm_expand_conv3x3_b64_28x28x512_to_512.md"),
+    ("dw3x3_b64_112x112x192_s1", "depthwise_lut"): (2.000 * 342889 * 1024 + 1.000 * 602112 * 1024,
+                                                    "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
+    ("dw3x3_b64_112x112x192_s2", "depthwise_lut"): (2.000 * 321245 * 1024 + 1.000 * 150528 * 1024,
+                                                    "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
 }
 
 
@@ -334,6 +339,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--codes", default="uniform", choices=["uniform", "halfnormal"])
+    ap.add_argument("--preexpand", type=int, default=0, choices=[-1, 0, 1],
+                    help="which dense layers run out of pre-expanded rows (axc_set_preexpand): 0 = the planner's "
+                         "choice, 1 = all that can, -1 = none (every layer expands its table rows inside every tile)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-layers", action="store_true", help="leave the `layers` array out (profiler runs)")
@@ -370,6 +378,7 @@ def main():
     import __graft_entry__ as entry
     pkg = entry.load_package()
     from tf_approximate_amd import ops, synth
+    ops.set_preexpand(args.preexpand)
 
     if args.network:
         r = measure_network(pkg, args.network, args.steps, args.warmup, args.fused_layers)
@@ -432,7 +441,7 @@ def main():
     achieved = lookups / (main_ms * 1e-3)
     ceil = Ceilings(ops)
     hbm_bytes = 4 * (x.size + y.numel()) + 4 * f.size + 131072
-    traffic, traffic_source = PROFILED_TRAFFIC.get(args.workload, (None, None))
+    traffic, traffic_source = PROFILED_TRAFFIC.get((args.workload, main_kernel), (None, None))
     if depthwise:
         # K = kh*kw is too small for LDS reuse: 8 bytes of HBM per output element against 9 lookups, HBM-bound
         roofline = {
@@ -527,7 +536,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "input": list(xs), "filter": list(fs), "strides": list(strides),
                    "padding": "SAME", "activation_codes": args.codes, "table": "clamp(a*b+U(-64,64))",
-                   "lookups": lookups},
+                   "lookups": lookups, "preexpand": args.preexpand},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "kernels_ms": {k: round(v, 4) for k, v in sorted(kms.items())},
