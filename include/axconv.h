@@ -143,7 +143,7 @@ int axc_qint32_range_for_multiplication(float min_a, float max_a, float min_b, f
 int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6]);
 /* Pins the tile width the planner uses (16, 32 or 64 columns; 0 = its own choice, the default), process-wide, for
  * tests and timing of the wider-tile kernel variants.  The environment variable AXC_TILE_COLUMNS gives the initial
- * value and is read once, when the library is loaded.  This is the library's only setting; a workspace query and
+ * value and is read once, when the library is loaded.  Like axc_set_preexpand it is process-wide; a workspace query and
  * the launch it is for must see the same value. */
 int axc_set_tile_columns(int columns);
 /* Layers with many output pixels per filter element (16-column tiles, no K split, an even number of channel quads,
