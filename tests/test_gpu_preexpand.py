@@ -98,6 +98,38 @@ def test_layer_entry_point_on_preexpanded_rows(pkg, oracle, forced):
     assert refimpl.linf_rel(y, y_ref) <= 1e-5
 
 
+def test_codes_and_tf1_entry_points_on_preexpanded_rows(pkg, oracle, forced):
+    """uint8 codes in, int32 sums out (axc_conv2d_codes_acc_i32), and the tf1 integer op with its own padding origin."""
+    from tf_approximate_amd import ops
+    rng = np.random.default_rng(8)
+    table_np = pkg.synth.table_random(21)
+    table = pkg.TruthTable(table_np)
+    for xs, fs, strides, padding, zp in [((1, 13, 13, 32), (3, 3, 32, 64), (2, 2), "SAME", 0),
+                                         ((3, 6, 6, 16), (1, 1, 16, 48), (1, 1), "VALID", 255),
+                                         ((2, 11, 9, 16), (1, 1, 16, 20), (2, 3), "SAME", 9)]:
+        qa = rng.integers(0, 256, xs).astype(np.uint8)
+        qb = rng.integers(0, 256, fs).astype(np.uint8)
+        forced.profile_reset()
+        acc = ops.conv2d_codes_acc_i32(table, torch.from_numpy(qa).to(gpu_util.dev()),
+                                       torch.from_numpy(qb).to(gpu_util.dev()), zp,
+                                       (1, strides[0], strides[1], 1), padding).cpu().numpy()
+        assert _ran_px(forced), (xs, fs)
+        patches = refimpl.gather_patches(qa, zp, fs[0], fs[1], strides, padding, (1, 1))
+        n, oh, ow = patches.shape[:3]
+        want = oracle.lut_gemm_codes(table_np, patches.reshape(n * oh * ow, -1), qb.reshape(-1, fs[3]))
+        assert np.array_equal(acc.reshape(n * oh * ow, fs[3]), want)
+    xs, fs, stride, padding, mm = (2, 7, 7, 256), (3, 3, 256, 16), 1, "SAME", (-1.0, 1.0, -0.5, 0.5)
+    x = rng.integers(0, 256, size=xs).astype(np.uint8)
+    f = rng.integers(0, 256, size=fs).astype(np.uint8)
+    forced.profile_reset()
+    out, _, _ = ops.ax_conv2d(torch.from_numpy(x).to(gpu_util.dev()), torch.from_numpy(f).to(gpu_util.dev()), *mm,
+                              [1, stride, stride, 1], padding, table)
+    assert _ran_px(forced)
+    off_in = ops.float_to_quantized_unclamped_quint8(0.0, mm[0], mm[1])
+    off_f = ops.float_to_quantized_unclamped_quint8(0.0, mm[2], mm[3])
+    assert np.array_equal(out.cpu().numpy(), oracle.axconv2d_tf1(table_np, x, f, off_in, off_f, stride, padding))
+
+
 def test_workspace_without_room_for_the_rows_still_serves(pkg, forced):
     """The workspace query counts the pre-expanded rows; the allocation-free entry point has 32 MiB and runs a layer
     whose rows alone take 128 MiB without them - same bits."""

@@ -116,8 +116,8 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
     const rsrc_t e_rsrc = make_rsrc(p.px_rows, p.px_bytes);
 
     // Tiles in blocks of kPxBlockCols column tiles: inside a block row tile after row tile, the column tile fastest.
-    // Workgroups with neighbouring indices sit on one XCD (own L2) and work on neighbouring tiles: the same few
-    // column tiles (same pre-expanded rows) of a few row tiles (same activations).
+    // The workgroups of an XCD (own L2) work on neighbouring tiles at the same time: the same few column tiles (same
+    // pre-expanded rows) of a few row tiles (same activations).
     auto decode = [&](const int tile, int &rt, int &ct) __attribute__((always_inline)) {
         const int per_block = n_row * kPxBlockCols;
         const int cb = tile / per_block;
@@ -127,9 +127,22 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
         rt = in_block / w;
         ct = cb * kPxBlockCols + in_block - rt * w;
     };
+    // Workgroups are handed to the 8 XCDs round-robin.  Each XCD gets one contiguous eighth of the tiles and its
+    // workgroups walk it side by side (workgroup i of the XCD takes its tiles i, i + 32, ...): an XCD stays with the
+    // same few column blocks for the whole launch, so their rows are fetched into its L2 once.
     const int G = (int)gridDim.x;
-    const int wg = (G & 7) == 0 ? ((int)blockIdx.x & 7) * (G >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
-    if (p.stagger_sleeps && ((wg / (n_col < kPxBlockCols ? n_col : kPxBlockCols)) & 1))
+    int tile_first, tile_end, tile_step;
+    if ((G & 7) == 0) {
+        const int xcd = (int)blockIdx.x & 7, i = (int)blockIdx.x >> 3;
+        tile_first = (int)((int64_t)ntiles * xcd / 8) + i;
+        tile_end = (int)((int64_t)ntiles * (xcd + 1) / 8);
+        tile_step = G >> 3;
+    } else {
+        tile_first = (int)blockIdx.x;
+        tile_end = ntiles;
+        tile_step = G;
+    }
+    if (p.stagger_sleeps && ((tile_first / (n_col < kPxBlockCols ? n_col : kPxBlockCols)) & 1))
         for (int i = 0; i < p.stagger_sleeps; ++i)
             __builtin_amdgcn_s_sleep(127);
 
@@ -145,19 +158,19 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
                 e_rsrc, (__attribute__((address_space(3))) void *)(lds_px + edst + j * 1024u), 16, (int)l16,
                 (int)(eoff + j * 1024u), 0, 0);
     };
-    if (wg < ntiles) {
+    if (tile_first < tile_end) {
         int rt0, ct0;
-        decode(wg, rt0, ct0);
+        decode(tile_first, rt0, ct0);
         load_first_fill(ct0);
     }
-    for (int tile = wg; tile < ntiles; tile += G) {
+    for (int tile = tile_first; tile < tile_end; tile += tile_step) {
         int rt, ct;
         decode(tile, rt, ct);
         int ct_next = ct;
-        const bool has_next = tile + G < ntiles;
+        const bool has_next = tile + tile_step < tile_end;
         if (has_next) {
             int rt_next;
-            decode(tile + G, rt_next, ct_next);
+            decode(tile + tile_step, rt_next, ct_next);
         }
         const TileRows t = tile_rows_of<R>(p, rt, wave);
         if (rt != prev_rt) {
