@@ -25,7 +25,7 @@ CASES = [
     ((1, 12, 11, 16), (3, 3, 16, 24), (1, 1), (1, 1), "SAME"),    # 18 fills (even), two column tiles
     ((3, 17, 13, 16), (3, 3, 16, 30), (2, 2), (1, 1), "VALID"),   # columns not a multiple of four: untransposed store
     ((2, 20, 20, 24), (5, 5, 24, 7), (1, 1), (1, 1), "SAME"),     # fewer than 16 columns
-    ((2, 21, 19, 6), (3, 3, 6, 20), (1, 2), (2, 1), "SAME"),      # 6 channels in two quads, dilation, mixed strides
+    ((2, 21, 19, 6), (3, 3, 6, 20), (1, 2), (2, 2), "SAME"),      # 6 channels in two quads, dilation, mixed strides
     ((1, 40, 40, 32), (1, 1, 32, 100), (1, 1), (1, 1), "SAME"),   # seven column tiles: two blocks of the tile order
     ((70, 9, 9, 8), (3, 3, 8, 24), (2, 2), (1, 1), "VALID"),      # many small images
     ((9, 60, 60, 8), (1, 1, 8, 160), (1, 1), (1, 1), "SAME"),     # 8 row tiles x 10 column tiles

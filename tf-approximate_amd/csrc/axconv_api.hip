@@ -472,12 +472,14 @@ struct DenseWorkspace {
 };
 
 // sub_bytes: room for the pixels a strided 1x1 filter reads, gathered into a dense tensor (see prepare_dense)
-DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan, size_t sub_bytes)
+DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan, size_t sub_bytes, int flat_row_bytes)
 {
     DenseWorkspace w;
     size_t off = 0;
     w.sub_off = off; off += align_up(sub_bytes);
-    w.xq_off = off; off += align_up(((size_t)g.N * g.H + 1) * g.C4 * g.W * 4); // + the zero-point row
+    w.xq_off = off;   // + the zero-point row; the flat layout's last quad may reach a few bytes past its row
+    off += align_up(flat_row_bytes ? ((size_t)g.N * g.H + 1) * flat_row_bytes + 16
+                                   : ((size_t)g.N * g.H + 1) * g.C4 * g.W * 4);
     w.psum_off = off; off += align_up((size_t)g.M * 4); // patch sums: one float per output pixel
     w.wq_off = off; off += align_up((size_t)plan.n_col_tiles * plan.fills * 64 * 2);
     w.fsum_off = off; off += align_up((size_t)g.Co * 4);
@@ -496,8 +498,10 @@ DenseWorkspace dense_workspace(const ConvGeom &g, const DensePlan &plan, size_t 
 
 struct PreparedDense {
     axc_conv2d_dims dims;
-    ConvGeom g;          // what the kernels see
+    ConvGeom g;          // what the pre-pass kernels see
     ConvGeom g_full;     // the layer as given (differs from g when the input is subsampled first)
+    ConvGeom gk;         // what the planner and the LUT-GEMM kernels see (differs from g in the flat layout)
+    int flat_row_bytes;  // > 0: xq in the flat layout, rows of this many bytes
     bool subsample;
     DensePlan plan;
     DenseWorkspace ws;
@@ -511,6 +515,7 @@ struct PreparedDense {
 // with their own padding origin).
 int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_subsample = true, int element_bytes = 4)
 {
+    const bool allow_flat = allow_subsample;   // both are for callers that leave the padding origin to the library
     int rc = geometry(desc, &pd->dims);
     if (rc != AXC_OK)
         return rc;
@@ -534,8 +539,29 @@ int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_sub
         pd->g.sh = pd->g.sw = 1;
         sub_bytes = (size_t)pd->g.M * pd->g.C * element_bytes;
     }
-    pd->plan = make_plan(pd->g, device_cus());
-    pd->ws = dense_workspace(pd->g, pd->plan, sub_bytes);
+    // Channel counts that are no multiple of four (3-channel stems) would pad every pixel to whole quads: a quarter
+    // of a 3-channel layer's lookups would hit the null weight.  With a filter dilation of 1 along the row, the KW * C
+    // codes under one filter row are contiguous in a pixel-major byte layout instead, and are cut into quads as one
+    // run: 21 -> 24 slots per row of a 7x7x3 filter where quads per pixel give 28.  The kernels then see a filter of
+    // KH taps over ceil(KW * C / 4) quads and read their activation dwords at byte granularity.  Not with a
+    // caller-defined padding origin (it may be negative).
+    pd->gk = pd->g;
+    pd->flat_row_bytes = 0;
+    {
+        const ConvGeom &g = pd->g;
+        const int run = g.KW * g.C, quads = (run + 3) / 4;
+        const int64_t row_bytes = std::max<int64_t>((int64_t)(g.pw + g.W) * g.C, (int64_t)(g.OW - 1) * g.sw * g.C + 4 * quads);
+        const int64_t rb4 = (row_bytes + 3) & ~(int64_t)3;
+        if (allow_flat && !pd->subsample && (g.C & 3) != 0 && g.dw == 1 && g.pw >= 0 && quads < g.KW * g.C4 &&
+            ((int64_t)g.N * g.H + 2) * rb4 < ((int64_t)1 << 31)) {
+            pd->flat_row_bytes = (int)rb4;
+            pd->gk.KW = 1;
+            pd->gk.C = run;       // the filter as [KH][KW * C][Co]
+            pd->gk.C4 = quads;
+        }
+    }
+    pd->plan = make_plan(pd->gk, device_cus());
+    pd->ws = dense_workspace(pd->g, pd->plan, sub_bytes, pd->flat_row_bytes);
     return AXC_OK;
 }
 
@@ -623,14 +649,23 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         else
             input = static_cast<const float *>(sub);
     }
+    const bool flat = pd.flat_row_bytes > 0;
+    const ConvGeom &gk = pd.gk;   // the layer as the LUT-GEMM kernels and the filter packing see it
     bool quantized_by_patch_sums = false, filter_done = false;
     if (out_f && !codes_mode) {
         ProfScope ps("patch_sums", stream);   // carries the filter pre-pass along when it can
         const FilterJob job = {filter, filter_codes, &pd.plan, tq_f, wq, fsum};
-        AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, &job,
-                                  &filter_done));
+        if (flat)   // the flat layout is written by its own pass below
+            AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream));
+        else
+            AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, &job,
+                                      &filter_done));
     }
-    if (codes_mode) {
+    if (flat) {
+        ProfScope ps("quantize_flat_rows", stream);
+        AXC_HIP(launch_quantize_flat_rows(input, codes_mode ? input_codes : nullptr, g, g.pw, pd.flat_row_bytes, tq_in,
+                                          lq_dev, reinterpret_cast<uint8_t *>(xq), stream));
+    } else if (codes_mode) {
         ProfScope ps("codes_relayout", stream);
         AXC_HIP(launch_codes_relayout(input_codes, g, zp4, xq, stream));
     } else if (!quantized_by_patch_sums) {
@@ -639,12 +674,14 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     }
     if (!filter_done) {
         ProfScope ps("filter_pack", stream);
-        AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, g, pd.plan, tq_f, lq_dev, wq,
+        AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, gk, pd.plan, tq_f, lq_dev, wq,
                                    (out_f && !codes_mode) ? fsum : nullptr, stream));
     }
 
     DenseParams p;
-    p.g = g;
+    p.g = gk;
+    p.g.ph = g.ph;   // a caller's own padding origin (never with the flat layout)
+    p.g.pw = g.pw;
     p.plan = pd.plan;
     p.xq = xq;
     p.psum = psum;
@@ -679,7 +716,21 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         p.px_rows = rows;
         p.px_bytes = (uint32_t)pd.ws.px_bytes;
     }
-    p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
+    if (flat) {
+        p.xq_bytes = (uint32_t)((size_t)g.N * g.H * pd.flat_row_bytes);
+        p.row_step = pd.flat_row_bytes;
+        p.addr_unit = 1;
+        p.quad_bytes = 4;
+        p.zp_tail_bytes = (uint32_t)pd.flat_row_bytes + 16;
+        p.flat_col_bytes = g.sw * g.C;
+    } else {
+        p.xq_bytes = (uint32_t)((size_t)g.N * g.H * g.C4 * g.W * 4);
+        p.row_step = g.C4 * g.W;
+        p.addr_unit = 4;
+        p.quad_bytes = (uint32_t)g.W * 4u;
+        p.zp_tail_bytes = (uint32_t)g.C4 * (uint32_t)g.W * 4u;
+        p.flat_col_bytes = 0;
+    }
     p.wq_bytes = (uint32_t)((size_t)pd.plan.n_col_tiles * pd.plan.fills * 128);
     {
         // Short-K layers with many tiles per workgroup (1x1 with few channels on large images) spend a quarter of

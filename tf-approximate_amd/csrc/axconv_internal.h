@@ -104,6 +104,15 @@ struct DenseParams {
     int stagger_sleeps;          // s_sleep(127) periods by which every second group of workgroups starts late (0: none)
     const uint16_t *px_rows;     // pre-expanded rows [n_col_tiles][fills / 2][256][128] (lutgemm_px_kernel only)
     uint32_t px_bytes;
+    // Addressing of xq.  Usual layout: dwords of four channels, [N][H][C4][W].  Flat layout (channel counts that are
+    // no multiple of four, see prepare_dense): bytes, [N][H][row], a row = the pixels' channels one after the other
+    // with the horizontal padding written out; g then describes a filter of KH taps whose "channels" are the
+    // KW * C bytes a filter row covers.
+    int row_step;                // between input rows, in address units
+    int addr_unit;               // bytes per address unit: 4 (dwords) or 1 (flat)
+    uint32_t quad_bytes;         // between the channel quads that one tap of a pixel reads
+    uint32_t zp_tail_bytes;      // size of the zero-point row behind xq
+    int flat_col_bytes;          // flat: bytes between horizontally neighbouring output pixels (sw * C); 0 = usual layout
 };
 
 struct DepthwiseParams {
@@ -199,6 +208,11 @@ hipError_t launch_subsample(const void *in, int element_bytes, int N, int H, int
                             void *out, hipStream_t stream);
 hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32_t zp4, uint32_t *xq,
                                  hipStream_t stream);
+// Flat layout of xq: rows of row_bytes bytes, pad_left pixels of the zero-point code, the W pixels' codes, zero-point
+// codes up to the end of the row; one more row of zero-point codes behind the last image.  From floats (x) or codes.
+hipError_t launch_quantize_flat_rows(const float *x, const uint8_t *codes, const ConvGeom &g, int pad_left,
+                                     int row_bytes, const TensorQuant &tq, const LayerQuant *lq_dev, uint8_t *xq,
+                                     hipStream_t stream);
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
                               const DensePlan &plan, const TensorQuant &tq, const LayerQuant *lq_dev,
                               uint16_t *wq, float *fsum, hipStream_t stream);

@@ -123,10 +123,9 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
     const int nct_v = p.plan.n_col_tiles * p.plan.k_splits;
     const int ntiles = p.plan.n_row_tiles * nct_v;
     const int fills_all = p.plan.fills;
-    const int rowstep = g.C4 * g.W; // dwords between input rows in xq
     // xq ends with one extra input row filled with the zero-point code: taps outside the image read it
     const uint32_t zp_row = p.xq_bytes;
-    const rsrc_t xq_rsrc = make_rsrc(p.xq, p.xq_bytes + (uint32_t)rowstep * 4u);
+    const rsrc_t xq_rsrc = make_rsrc(p.xq, p.xq_bytes + p.zp_tail_bytes);
     const rsrc_t wq_rsrc = make_rsrc(p.wq, p.wq_bytes);
     const rsrc_t tab_rsrc = make_rsrc(p.tableT, (uint32_t)kTableAllocBytes);
     (void)taps;
@@ -166,9 +165,9 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
         int cur_fill = 0, cur_sub = f0 % SUBS;
         int cur_q = (f0 / SUBS) % g.C4, cur_kh = (f0 / SUBS / g.C4) / g.KW, cur_kw = (f0 / SUBS / g.C4) % g.KW;
         uint32_t idx_tap[R];   // byte offset in xq of quad 0 of the current tap (the zero-point row outside)
-        auto tap_setup = [&]() { tap_offsets<R>(g, park, cur_kh, cur_kw, zp_row, idx_tap); };
+        auto tap_setup = [&]() { tap_offsets<R>(p, park, cur_kh, cur_kw, zp_row, idx_tap); };
         auto load_acts = [&](uint32_t (&dst)[R]) {
-            const uint32_t qoff = (uint32_t)(cur_q * g.W * 4); // scalar: channel quad inside the pixel row
+            const uint32_t qoff = (uint32_t)cur_q * p.quad_bytes; // scalar: channel quad inside the pixel row
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 dst[r] = ld_u32(xq_rsrc, idx_tap[r], qoff);
@@ -281,7 +280,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_expand_kernel(const Den
             constexpr int BUF = decltype(buf_tag)::value;
             const int fcodes = pcur + 3 < fills_left ? pcur + 3 : fills_left - 1;
             const uint32_t cso = wq_tile + (uint32_t)fcodes * 128u;
-            const uint32_t qoff = (uint32_t)(cur_q * g.W * 4);
+            const uint32_t qoff = (uint32_t)cur_q * p.quad_bytes;
             phase_body<NT, BUF>(acc, act_cur, act_next, idx_tap, codes, k, nr_s,
                                 __builtin_amdgcn_readfirstlane(shift_cur), tab_rsrc, wq_rsrc, xq_rsrc,
                                 __builtin_amdgcn_readfirstlane(cso), __builtin_amdgcn_readfirstlane(qoff));

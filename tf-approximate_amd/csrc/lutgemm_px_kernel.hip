@@ -108,11 +108,11 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
     const int ntiles = n_row * n_col;
     const int F = p.plan.fills / 2;                 // pre-expanded fills over K
     const int qpairs = g.C4 / 2;                    // fills per tap
-    const uint32_t quad_bytes = (uint32_t)g.W * 4u; // between the channel quads of a pixel in xq
+    const uint32_t quad_bytes = p.quad_bytes;        // between the channel quads of a pixel in xq
     const uint32_t dlf = upper ? quad_bytes : 0u;   // this lane's FIRST dword is the pair's second quad if swapped
     const uint32_t dls = upper ? 0u : quad_bytes;
     const uint32_t zp_row = p.xq_bytes;             // one extra input row of the zero-point code behind xq
-    const rsrc_t xq_rsrc = make_rsrc(p.xq, p.xq_bytes + (uint32_t)(g.C4 * g.W) * 4u);
+    const rsrc_t xq_rsrc = make_rsrc(p.xq, p.xq_bytes + p.zp_tail_bytes);
     const rsrc_t e_rsrc = make_rsrc(p.px_rows, p.px_bytes);
 
     // Tiles in blocks of kPxBlockCols column tiles: inside a block row tile after row tile, the column tile fastest.
@@ -182,14 +182,14 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
         // ---- activation cursor: (tap, quad pair) of the fill whose activations are fetched next ----
         int cur_fill = 0, cur_qp = 0, cur_kh = 0, cur_kw = 0;
         uint32_t idx_tap[R];
-        tap_offsets<R>(g, park, 0, 0, zp_row, idx_tap);
+        tap_offsets<R>(p, park, 0, 0, zp_row, idx_tap);
         auto advance_cursor = [&]() __attribute__((always_inline)) {
             ++cur_fill;
             if (++cur_qp == qpairs) {
                 cur_qp = 0;
                 if (++cur_kw == g.KW) { cur_kw = 0; ++cur_kh; }
                 if (cur_fill < F)
-                    tap_offsets<R>(g, park, cur_kh, cur_kw, zp_row, idx_tap);
+                    tap_offsets<R>(p, park, cur_kh, cur_kw, zp_row, idx_tap);
             }
         };
         uint32_t fA[R], sA[R], fB[R], sB[R];

@@ -50,14 +50,14 @@ __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, i
 
 // Per-pixel geometry of this lane's R pixels, parked in LDS in slots private to the thread (park[slot *
 // kDenseThreads]) and read back only when the tap changes: slot 2r = dword index in xq of tap (0, 0), channel
-// quad 0 (may point outside the image), slot 2r+1 = input coordinates of tap (0, 0) as (ih0 << 16) | (iw0 & 0xffff),
+// quad 0 in address units (may point outside the image), slot 2r+1 = input coordinates of tap (0, 0) as (ih0 << 16) | (iw0 & 0xffff),
 // 0x80000000 for a pixel that does not exist.  Returns the number of this lane's pixels whose wavefront-row exists
 // (a prefix of the R; the same in every lane of the wavefront).
 template <int R>
 __device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const TileRows &t, int lane, uint32_t *park)
 {
     const ConvGeom &g = p.g;
-    const int rowstep = g.C4 * g.W;
+    const int rowstep = p.row_step;
     uint32_t nr = 0;
     // (n, oh, ow) of this lane's first pixel by division; its further pixels lie a fixed number of output
     // pixels apart (four wavefront-rows), so they follow by adding that step's (n, oh, ow) with carries
@@ -82,8 +82,11 @@ __device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const Ti
         const int64_t wrow = t.row0 + (int64_t)(t.wr_base + r * (kDenseWaves / 2)) * 64;
         nr += (wrow < t.row_end && wrow < t.wr_end) ? 1u : 0u;
         const bool valid = wrow + lane < t.row_end && wrow < t.wr_end;
-        const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
-        park[(2 * r) * kDenseThreads] = valid ? (uint32_t)((n * g.H + ih0) * rowstep + iw0) : 0u;
+        // flat layout: the horizontal padding is part of the row, so the column of tap (0, 0) is ow * sw pixels in
+        // and never outside (stored as column 0)
+        const int ih0 = oh * g.sh - g.ph, iw0 = p.flat_col_bytes ? 0 : ow * g.sw - g.pw;
+        const int col = p.flat_col_bytes ? ow * p.flat_col_bytes : iw0;
+        park[(2 * r) * kDenseThreads] = valid ? (uint32_t)((n * g.H + ih0) * rowstep + col) : 0u;
         park[(2 * r + 1) * kDenseThreads] = valid ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
         // the next pixel of this lane: p.step_* = (n, oh, ow) of 64 * kDenseWaves / 2 output pixels
         ow += p.step_ow;
@@ -99,11 +102,12 @@ __device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const Ti
 
 // byte offset in xq of quad 0 of tap (kh, kw) for each of the lane's pixels; the zero-point row outside the image
 template <int R>
-__device__ __forceinline__ void tap_offsets(const ConvGeom &g, const uint32_t *park, int kh, int kw, uint32_t zp_row,
+__device__ __forceinline__ void tap_offsets(const DenseParams &p, const uint32_t *park, int kh, int kw, uint32_t zp_row,
                                             uint32_t (&idx_tap)[R])
 {
+    const ConvGeom &g = p.g;
     const int dh = kh * g.dh, dw = kw * g.dw;
-    const int tap_off = dh * g.C4 * g.W + dw;
+    const int tap_off = dh * p.row_step + dw;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int32_t pb = (int32_t)park[(2 * r) * kDenseThreads];
@@ -111,7 +115,7 @@ __device__ __forceinline__ void tap_offsets(const ConvGeom &g, const uint32_t *p
         const int ih = (hw >> 16) + dh;
         const int iw = (int)(int16_t)(hw & 0xffff) + dw;
         const bool inb = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-        idx_tap[r] = inb ? (uint32_t)((pb + tap_off) * 4) : zp_row;
+        idx_tap[r] = inb ? (uint32_t)((pb + tap_off) * p.addr_unit) : zp_row;
     }
 }
 

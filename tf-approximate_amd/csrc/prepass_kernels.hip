@@ -1560,6 +1560,52 @@ hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, 
     return hipGetLastError();
 }
 
+// Flat layout of the quantized input for channel counts that are no multiple of four: one thread per dword of xq.
+// Byte b of row r (r = image * H + input row; row N * H is the zero-point row that taps outside the image read)
+// is the code of channel b % C of pixel b / C - pad_left, the zero-point code where that pixel lies outside the
+// image or b lies behind the last pixel.
+__global__ void __launch_bounds__(256) quantize_flat_rows_kernel(const float *__restrict__ x,
+                                                                 const uint8_t *__restrict__ codes, int64_t rows,
+                                                                 int W, int C, int pad_left, int row_bytes,
+                                                                 const TensorQuant tq,
+                                                                 const LayerQuant *__restrict__ lq_dev,
+                                                                 uint32_t *__restrict__ xq)
+{
+    const TensorQuant qt = lq_dev ? lq_dev->in : tq;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // dword index
+    const int dwords_per_row = row_bytes / 4;
+    if (i >= (rows + 1) * dwords_per_row)
+        return;
+    const int64_t r = i / dwords_per_row;
+    const int b0 = (int)(i - r * dwords_per_row) * 4;
+    const uint32_t zp = qt.zp4 & 0xffu;
+    uint32_t word = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int b = b0 + k;
+        const int px = b / C, c = b - px * C, w = px - pad_left;
+        uint32_t code = zp;
+        if (r < rows && (unsigned)w < (unsigned)W) {
+            const int64_t src = (r * W + w) * C + c;
+            code = codes ? phys_row(codes[src])
+                         : phys_row(quantize_code(fake_quant_value(x[src], qt), qt.offset, qt.inv_scale));
+        }
+        word |= code << (8 * k);
+    }
+    xq[i] = word;
+}
+
+hipError_t launch_quantize_flat_rows(const float *x, const uint8_t *codes, const ConvGeom &g, int pad_left,
+                                     int row_bytes, const TensorQuant &tq, const LayerQuant *lq_dev, uint8_t *xq,
+                                     hipStream_t stream)
+{
+    const int64_t rows = (int64_t)g.N * g.H;
+    const int64_t dwords = (rows + 1) * (row_bytes / 4);
+    hipLaunchKernelGGL(quantize_flat_rows_kernel, dim3(blocks_for(dwords, 256)), dim3(256), 0, stream, x, codes, rows,
+                       g.W, g.C, pad_left, row_bytes, tq, lq_dev, reinterpret_cast<uint32_t *>(xq));
+    return hipGetLastError();
+}
+
 hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
                                 hipStream_t stream)
 {
