@@ -86,8 +86,8 @@ PROFILED_TRAFFIC = {
                                                     "profiles/lutgemm_px_conv1x1_b64_56x56x64_to_256.md"),
     ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 466561.3 * 1024 + 1.000 * 471098.3 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
-    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_expand"): (2.000 * 9530.0 * 1024 + 1.000 * 244804.3 * 1024,
-                                                          "profiles/lutgemm_expand_conv7x7s2_b64_224x224x3_to_64.md"),
+    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 92811.5 * 1024 + 1.000 * 259828.2 * 1024,
+                                                      "profiles/lutgemm_px_conv7x7s2_b64_224x224x3_to_64.md"),
     ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51682.9 * 1024 + 1.000 * 106672.4 * 1024,
                                                          "profiles/lutgemm_expand_conv3x3_b64_28x28x512_to_512.md"),
     ("dw3x3_b64_112x112x192_s1", "depthwise_lut"): (2.000 * 342889 * 1024 + 1.000 * 602112 * 1024,
