@@ -653,18 +653,21 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     const ConvGeom &gk = pd.gk;   // the layer as the LUT-GEMM kernels and the filter packing see it
     bool quantized_by_patch_sums = false, filter_done = false;
     if (out_f && !codes_mode) {
-        ProfScope ps("patch_sums", stream);   // carries the filter pre-pass along when it can
+        ProfScope ps(flat ? "patch_sums_flat" : "patch_sums", stream);   // carries the filter pre-pass along when it can
         const FilterJob job = {filter, filter_codes, &pd.plan, tq_f, wq, fsum};
-        if (flat)   // the flat layout is written by its own pass below
-            AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream));
+        if (flat)   // the patch sums write the flat layout where they hold the rows anyway, else the pass below does
+            AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, nullptr,
+                                      nullptr, pd.flat_row_bytes));
         else
             AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, &job,
                                       &filter_done));
     }
-    if (flat) {
+    if (flat && !quantized_by_patch_sums) {
         ProfScope ps("quantize_flat_rows", stream);
         AXC_HIP(launch_quantize_flat_rows(input, codes_mode ? input_codes : nullptr, g, g.pw, pd.flat_row_bytes, tq_in,
                                           lq_dev, reinterpret_cast<uint8_t *>(xq), stream));
+    } else if (flat) {
+        // written by the patch-sum launch
     } else if (codes_mode) {
         ProfScope ps("codes_relayout", stream);
         AXC_HIP(launch_codes_relayout(input_codes, g, zp4, xq, stream));

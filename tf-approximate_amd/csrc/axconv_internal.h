@@ -199,7 +199,8 @@ struct FilterJob {
 // filter_job / filter_done: it may also do the filter pre-pass (then *filter_done is set).
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
                              float *psum, hipStream_t stream, uint32_t *xq_fused = nullptr, bool *fused = nullptr,
-                             const FilterJob *filter_job = nullptr, bool *filter_done = nullptr);
+                             const FilterJob *filter_job = nullptr, bool *filter_done = nullptr,
+                             int flat_row_bytes = 0);   // > 0: a fused xq is written in the flat layout
 hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
                               float *partials, LayerQuant *lq_dev, hipStream_t stream);
 constexpr int kMinMaxBlocks = 2048;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch

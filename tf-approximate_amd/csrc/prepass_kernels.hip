@@ -463,12 +463,15 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
 __global__ void __launch_bounds__(1024) patch_sums_smallc_kernel(const float *__restrict__ x, const ConvGeom g,
                                                                   const int rb, const int in_rows, const TensorQuant tq,
                                                                   const LayerQuant *__restrict__ lq_dev,
-                                                                  float *__restrict__ psum, uint32_t *__restrict__ xq)
+                                                                  float *__restrict__ psum, uint32_t *__restrict__ xq,
+                                                                  const int flat_row_bytes, const int pad_left)
 {
+    // flat_row_bytes > 0: xq in the flat layout (see quantize_flat_rows_kernel), rows of that many bytes
     const TensorQuant qt = lq_dev ? lq_dev->in : tq;
+    const int zp_row_dwords = flat_row_bytes ? flat_row_bytes / 4 : g.C4 * g.W;
     if (xq && blockIdx.x == 0)
-        for (int i = threadIdx.x; i < g.C4 * g.W; i += blockDim.x)
-            xq[(int64_t)g.N * g.H * g.C4 * g.W + i] = qt.zp4;
+        for (int i = threadIdx.x; i < zp_row_dwords; i += blockDim.x)
+            xq[(int64_t)g.N * g.H * zp_row_dwords + i] = qt.zp4;
     extern __shared__ __align__(16) unsigned char ps_lds[];
     float *const rows = reinterpret_cast<float *>(ps_lds);
     const int t = threadIdx.x;
@@ -487,7 +490,27 @@ __global__ void __launch_bounds__(1024) patch_sums_smallc_kernel(const float *__
         rows[i] = (unsigned)ih < (unsigned)g.H ? fake_quant_value(x[((int64_t)n * g.H + ih) * row_floats + e], qt) : 0.0f;
     }
     __syncthreads();
-    if (xq) {
+    if (xq && flat_row_bytes) {
+        const int own_lo = oh0 * g.sh;           // owned input rows: [own_lo, own_hi)
+        const int own_hi = (oh0 + rb >= g.OH) ? g.H : (oh0 + rb) * g.sh;
+        const int per_row = flat_row_bytes / 4;  // one dword of the flat row per step
+        const uint32_t zp = qt.zp4 & 0xffu;
+        for (int i = t; i < (own_hi - own_lo) * per_row; i += blockDim.x) {
+            const int ro = i / per_row, d = i - ro * per_row;
+            const int ih = own_lo + ro;
+            const float *src = &rows[(ih - ih_first) * row_floats];
+            uint32_t packed = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int b = d * 4 + k, px = b / g.C, c = b - px * g.C, w = px - pad_left;
+                const uint32_t code = (unsigned)w < (unsigned)g.W
+                                          ? phys_row(quantize_code(src[w * g.C + c], qt.offset, qt.inv_scale))
+                                          : zp;
+                packed |= code << (8 * k);
+            }
+            xq[((int64_t)n * g.H + ih) * per_row + d] = packed;
+        }
+    } else if (xq) {
         const int own_lo = oh0 * g.sh;           // owned input rows: [own_lo, own_hi)
         const int own_hi = (oh0 + rb >= g.OH) ? g.H : (oh0 + rb) * g.sh;
         const int per_row = g.C4 * g.W;
@@ -1358,13 +1381,15 @@ static void choose_band(const ConvGeom &g, int64_t row_bytes, int sum_blocks, in
 
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
                              float *psum, hipStream_t stream, uint32_t *xq_fused, bool *fused,
-                             const FilterJob *filter_job, bool *filter_done)
+                             const FilterJob *filter_job, bool *filter_done, int flat_row_bytes)
 {
     if (fused)
         *fused = false;
     if (filter_done)
         *filter_done = false;
     const bool vec = (g.C & 3) == 0 && ((uintptr_t)x & 15) == 0;
+    if (flat_row_bytes && vec)   // the flat layout belongs to channel counts that are no multiple of four
+        return hipErrorInvalidValue;
     if (vec && g.OW <= 1024) {
         // largest band of output rows whose input rows fit in 96 KiB of LDS and whose pixels fit in one block,
         // but no larger than what still leaves every CU a few blocks
@@ -1477,7 +1502,7 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
             const int bands = (g.OH + rb - 1) / rb;
             hipLaunchKernelGGL(patch_sums_smallc_kernel, dim3((unsigned)((int64_t)g.N * bands)), dim3(threads),
                                (size_t)in_rows * row_bytes, stream, x, g, rb, in_rows, tq, lq_dev, psum,
-                               fuse ? xq_fused : nullptr);
+                               fuse ? xq_fused : nullptr, flat_row_bytes, g.pw);
             return hipGetLastError();
         }
     }
