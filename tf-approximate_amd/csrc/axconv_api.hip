@@ -374,14 +374,19 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
         const int64_t cap_wrows = (int64_t)kDenseWaves * R; // wavefront-rows (64 pixels each) per tile
         const int64_t total_wrows = (g.M + 63) / 64;
         const int64_t min_tiles = (total_wrows + cap_wrows - 1) / cap_wrows;
-        // candidate row-tile counts: the minimum, and counts that fill whole rounds of CUs
+        // candidate row-tile counts: the minimum, and counts that fill whole rounds of CUs, alone or together with
+        // a split of K
         std::vector<int64_t> cands{min_tiles};
         for (int64_t rounds = 1; rounds <= 48; ++rounds) {
-            int64_t n_row = (rounds * cus) / n_col;
-            if (n_row > min_tiles && n_row <= total_wrows)
-                cands.push_back(n_row);
-            if (n_row + 1 > min_tiles && n_row + 1 <= total_wrows)
-                cands.push_back(n_row + 1);
+            for (int split : {1, 2, 3, 4, 6, 8, 12, 16}) {
+                if (split > 1 && rounds > 2)
+                    break;
+                const int64_t n_row = (rounds * cus) / ((int64_t)n_col * split);
+                if (n_row > min_tiles && n_row <= total_wrows)
+                    cands.push_back(n_row);
+                if (split == 1 && n_row + 1 > min_tiles && n_row + 1 <= total_wrows)
+                    cands.push_back(n_row + 1);
+            }
         }
         if (total_wrows > min_tiles)
             cands.push_back(total_wrows);
@@ -403,8 +408,23 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
                 double cost = (double)rounds * ((double)fps * per_fill + 6000.0);
                 if (ks > 1) // the extra pass, and a margin: split only for a clear gain
                     cost = cost * 1.08 + 20000.0 + (double)(ks + 1) * (double)g.M * g.Co * 4.0 * 7e-4;
+                // The same tiles out of pre-expanded rows (16 columns, whole K, channel quads in pairs): a phase
+                // covers two fills and neither expands nor stages (fitted: 8 300 cycles at 13 wavefront-rows per
+                // SIMD, 2 900 at 2); the rows cost 512 bytes of memory per filter element, written once per call by
+                // one more launch (~6.5 us, then ~5 TB/s).
+                int px = 0;
+                if (px_possible && px_mode >= 0 && nt == 16 && ks == 1) {
+                    const double px_bytes = (double)n_col * (double)(fills / 2) * 65536.0;
+                    const double px_cost = (double)rounds * ((double)(fills / 2) * (1900.0 + per_simd * 530.0) + 12000.0) +
+                                           (6.5e-6 + px_bytes / 5e12) * 2.4e9;
+                    if (px_mode > 0 || px_cost < cost) {
+                        cost = px_cost;
+                        px = 1;
+                    }
+                }
                 if (cost < best_cost) {
                     best_cost = cost;
+                    best.px = px;
                     best.nt = nt;
                     best.rows_per_tile = (int)(wrows * 64);
                     best.n_row_tiles = (int)((total_wrows + wrows - 1) / wrows);
@@ -417,17 +437,6 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
                 }
             }
         }
-    }
-    // Pre-expanded rows: 16-column tiles over the whole K, channel quads in pairs.  They cost 512 bytes of memory per
-    // filter element, written once per call (one more launch: ~6.5 us, then ~5 TB/s) and read once per XCD; the lookup
-    // kernel then runs about an eighth faster (measured: 10-15 % at ~24 T lookups/s).  Worth it with many output
-    // pixels per filter element.
-    best.px = 0;
-    const size_t px_bytes = (size_t)best.n_col_tiles * (size_t)(best.fills / 2) * 65536;
-    if (px_mode >= 0 && best.nt == 16 && best.k_splits == 1 && (g.C4 & 1) == 0 && px_bytes <= kPxMaxBytes) {
-        const double lookups = (double)g.M * (double)best.fills * 4.0 * (double)best.n_col_tiles * 16.0;
-        const double gain_s = 0.12 * lookups / 24e12, cost_s = 6.5e-6 + (double)px_bytes / 5e12;
-        best.px = (px_mode > 0 || gain_s > cost_s) ? 1 : 0;
     }
     return best;
 }

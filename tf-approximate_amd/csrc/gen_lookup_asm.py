@@ -316,12 +316,22 @@ def emit_px(buf):
             st.ins("s_nop 0")
         return f
 
-    def act_load(r):         # both activation dwords of pixel r for the next fill
-        def f(st, state):
+    skips = [0]
+
+    def act_load(r):         # both activation dwords of pixel r for the next fill; skipped for a pixel the wavefront
+        def f(st, state):    # does not have (a gather costs the CU's address unit as much as 1 KiB of the fill)
+            label = None
+            if r > 0:
+                label = "Lskip%d_%%=" % skips[0]
+                skips[0] += 1
+                st.ins("s_cmp_lt_u32 %d, %%[nr]" % r)
+                st.ins("s_cbranch_scc0 %s" % label)
             st.ins("v_add_u32 v%d, %%[t%d], %%[dlf]" % (ADDR_BASE + 2, r))
             st.ins("buffer_load_dword %%[nf%d], v%d, %%[xq], %%[qoff] offen" % (r, ADDR_BASE + 2))
             st.ins("v_add_u32 v%d, %%[t%d], %%[dls]" % (ADDR_BASE + 3, r))
             st.ins("buffer_load_dword %%[ng%d], v%d, %%[xq], %%[qoff] offen" % (r, ADDR_BASE + 3))
+            if label:
+                st.label(label)
         return f
 
     aux = [e_load(j) for j in range(8)] + [act_load(r) for r in range(rows)]

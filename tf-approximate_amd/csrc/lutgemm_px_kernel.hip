@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
             int rt_next;
             decode(tile + tile_step, rt_next, ct_next);
         }
-        const TileRows t = tile_rows_of<R>(p, rt, wave);
+        const TileRows t = tile_rows_of<R, true>(p, rt, wave);
         if (rt != prev_rt) {
             prev_rt = rt;
             nr = park_geometry<R>(p, t, lane, park);
@@ -188,8 +188,8 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
             if (++cur_qp == qpairs) {
                 cur_qp = 0;
                 if (++cur_kw == g.KW) { cur_kw = 0; ++cur_kh; }
-                if (cur_fill < F)
-                    tap_offsets<R>(p, park, cur_kh, cur_kw, zp_row, idx_tap);
+                if (cur_fill < F)   // pixel 0's activations are fetched whether the wavefront has a pixel or not
+                    tap_offsets<R>(p, park, cur_kh, cur_kw, zp_row, idx_tap, nr_s > 1u ? nr_s : 1u);
             }
         };
         uint32_t fA[R], sA[R], fB[R], sB[R];

@@ -32,7 +32,7 @@ struct TileRows {
     int64_t wr_end;         // end of the pixels owned by this wavefront's half
     int wr_base;
 };
-template <int R>
+template <int R, bool EVEN_SMALL = false>
 __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, int wave)
 {
     TileRows t;
@@ -40,6 +40,10 @@ __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, i
     t.row_end = (t.row0 + p.plan.rows_per_tile < p.g.M) ? t.row0 + p.plan.rows_per_tile : p.g.M;
     const int wrows = (int)((t.row_end - t.row0 + 63) / 64);
     int wr_old = (wrows * kOldShare + 8) / 16;
+    // EVEN_SMALL: with up to one wavefront-row per wavefront, one each (for a kernel whose phase then lasts as long
+    // as the lookups of its slowest wavefront)
+    if (EVEN_SMALL && wrows <= kDenseWaves)
+        wr_old = wrows < kDenseWaves / 2 ? wrows : kDenseWaves / 2;
     wr_old = wr_old > 4 * R ? 4 * R : wr_old;
     wr_old = wr_old < wrows - 4 * R ? wrows - 4 * R : wr_old;
     const bool old_half = wave < kDenseWaves / 2;
@@ -100,16 +104,19 @@ __device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const Ti
     return nr;
 }
 
-// byte offset in xq of quad 0 of tap (kh, kw) for each of the lane's pixels; the zero-point row outside the image
+// byte offset in xq of quad 0 of tap (kh, kw) for each of the lane's pixels; the zero-point row outside the image.
+// live (the same for the whole wavefront): only the first `live` pixels are recomputed, the others keep what they hold.
 template <int R>
 __device__ __forceinline__ void tap_offsets(const DenseParams &p, const uint32_t *park, int kh, int kw, uint32_t zp_row,
-                                            uint32_t (&idx_tap)[R])
+                                            uint32_t (&idx_tap)[R], uint32_t live = R)
 {
     const ConvGeom &g = p.g;
     const int dh = kh * g.dh, dw = kw * g.dw;
     const int tap_off = dh * p.row_step + dw;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
+        if ((uint32_t)r >= live)
+            break;
         const int32_t pb = (int32_t)park[(2 * r) * kDenseThreads];
         const int32_t hw = (int32_t)park[(2 * r + 1) * kDenseThreads];
         const int ih = (hw >> 16) + dh;
