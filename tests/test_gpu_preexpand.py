@@ -4,7 +4,7 @@ The planner only picks it for layers with many output pixels, so the small cases
 axc_set_preexpand(1); every case also checks, from the library's own kernel timers, that this kernel is the one that
 ran.  Shapes cover one and many fills, odd and even fill counts (the two ways a tile hands LDS buffer 0 to the next
 tile), several tiles per workgroup, ragged row tiles, column counts that are not multiples of 16 or of 4, strides,
-dilation, padding taps, the layer entry point and the codes entry point."""
+dilation, padding taps, K cut over tiles, the layer entry point and the codes entry point."""
 import ctypes
 
 import numpy as np
@@ -56,6 +56,31 @@ def test_preexpanded_rows_vs_oracle(pkg, oracle, forced, case):
     y, acc = gpu_util.run_op(pkg, table, x, f, MM, strides, padding, dil)
     assert _ran_px(forced), case
     rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *MM, strides=strides, padding=padding, dilations=dil, threads=8)
+    assert rc == 0
+    assert np.array_equal(acc, acc_ref), case
+    assert refimpl.linf_rel(y, y_ref) <= 1e-5, case
+
+
+SPLIT_CASES = [
+    # few output pixels under a long K: the planner cuts K over tiles, each tile a whole number of pre-expanded fills
+    ((2, 8, 8, 64), (3, 3, 64, 32), (1, 1), "SAME"),
+    ((1, 14, 14, 256), (1, 1, 256, 64), (1, 1), "SAME"),
+    ((4, 7, 7, 128), (3, 3, 128, 48), (1, 1), "VALID"),
+    ((3, 9, 9, 40), (5, 5, 40, 20), (2, 2), "SAME"),          # 10 channel quads: a split starts inside a tap
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES, ids=[str(i) for i in range(len(SPLIT_CASES))])
+def test_preexpanded_rows_with_k_split_vs_oracle(pkg, oracle, forced, case):
+    xs, fs, strides, padding = case
+    plan = forced.conv2d_tile_plan(xs, fs, (1, strides[0], strides[1], 1), padding)
+    assert plan["k_splits"] > 1, plan
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=len(str(case)))
+    table = pkg.synth.table_random(17)
+    y, acc = gpu_util.run_op(pkg, table, x, f, MM, strides, padding)
+    prof = forced.profile_read()
+    assert _ran_px(forced) and "splitk_epilogue" in prof, (case, sorted(prof))
+    rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *MM, strides=strides, padding=padding, threads=8)
     assert rc == 0
     assert np.array_equal(acc, acc_ref), case
     assert refimpl.linf_rel(y, y_ref) <= 1e-5, case

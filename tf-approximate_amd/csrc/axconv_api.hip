@@ -398,25 +398,31 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
             // Splitting K over tiles keeps the tiles tall (many lookups per expanded fill) when M alone does not
             // give every CU a tile; the int32 partial sums then cost one more pass over (k_splits + 1) outputs.
             for (int ks : {1, 2, 3, 4, 6, 8, 12, 16}) {
-                if (want_px && (ks > 1 || nt != 16))
-                    break;  // pre-expanded rows are asked for wherever they are possible: 16 columns, whole K
-                const int fps = (fills + ks - 1) / ks;
+                if (want_px && nt != 16)
+                    break;  // pre-expanded rows are asked for wherever they are possible: 16 columns
+                int fps = (fills + ks - 1) / ks;
+                if (want_px && ks > 1)
+                    fps += fps & 1;   // a K split covers whole pre-expanded fills: pairs of fills
                 if (ks > 1 && (fps < 8 || (int64_t)(ks - 1) * fps >= fills))
                     continue;
                 const int64_t tiles = n_row * n_col * ks;
                 const int64_t rounds = (tiles + cus - 1) / cus;
                 double cost = (double)rounds * ((double)fps * per_fill + 6000.0);
-                if (ks > 1) // the extra pass, and a margin: split only for a clear gain
-                    cost = cost * 1.08 + 20000.0 + (double)(ks + 1) * (double)g.M * g.Co * 4.0 * 7e-4;
+                // the extra pass of a K split, and a margin: split only for a clear gain
+                const double split_cost = ks > 1 ? 20000.0 + (double)(ks + 1) * (double)g.M * g.Co * 4.0 * 7e-4 : 0.0;
+                if (ks > 1)
+                    cost = cost * 1.08 + split_cost;
                 // The same tiles out of pre-expanded rows (16 columns, whole K, channel quads in pairs): a phase
                 // covers two fills and neither expands nor stages (fitted: 8 300 cycles at 13 wavefront-rows per
                 // SIMD, 2 900 at 2); the rows cost 512 bytes of memory per filter element, written once per call by
                 // one more launch (~6.5 us, then ~5 TB/s).
                 int px = 0;
-                if (px_possible && px_mode >= 0 && nt == 16 && ks == 1) {
+                if (px_possible && px_mode >= 0 && nt == 16 && (ks == 1 || (fps & 1) == 0)) {
                     const double px_bytes = (double)n_col * (double)(fills / 2) * 65536.0;
-                    const double px_cost = (double)rounds * ((double)(fills / 2) * (1900.0 + per_simd * 530.0) + 12000.0) +
-                                           (6.5e-6 + px_bytes / 5e12) * 2.4e9;
+                    double px_cost = (double)rounds * ((double)(fps / 2) * (1900.0 + per_simd * 530.0) + 12000.0);
+                    if (ks > 1)
+                        px_cost = px_cost * 1.08 + split_cost;
+                    px_cost += (6.5e-6 + px_bytes / 5e12) * 2.4e9;
                     if (px_mode > 0 || px_cost < cost) {
                         cost = px_cost;
                         px = 1;
@@ -765,7 +771,10 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         int32_t *part = reinterpret_cast<int32_t *>(ws + pd.ws.part_off);
         p.out_f = nullptr;
         p.out_i = part;
-        {
+        if (use_px) {
+            ProfScope ps("lutgemm_px", stream);
+            AXC_HIP(launch_dense_px(p, true, stream));
+        } else {
             ProfScope ps("lutgemm_expand", stream);
             AXC_HIP(launch_dense(p, true, stream));
         }

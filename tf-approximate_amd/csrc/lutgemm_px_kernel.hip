@@ -104,9 +104,11 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
     const uint32_t l16 = (uint32_t)lane * 16u;
     uint32_t *const park = reinterpret_cast<uint32_t *>(lds_px + 2 * kPxFillBytes) + tid;
 
-    const int n_col = p.plan.n_col_tiles, n_row = p.plan.n_row_tiles;
+    // a tile = (row tile, column tile, K split); the K splits of a column tile count as further column tiles
+    const int n_col = p.plan.n_col_tiles * p.plan.k_splits, n_row = p.plan.n_row_tiles;
     const int ntiles = n_row * n_col;
     const int F = p.plan.fills / 2;                 // pre-expanded fills over K
+    const int Fs = p.plan.k_splits > 1 ? p.plan.fills_per_split / 2 : F;   // ... and per K split
     const int qpairs = g.C4 / 2;                    // fills per tap
     const uint32_t quad_bytes = p.quad_bytes;        // between the channel quads of a pixel in xq
     const uint32_t dlf = upper ? quad_bytes : 0u;   // this lane's FIRST dword is the pair's second quad if swapped
@@ -149,9 +151,11 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
     int prev_rt = -1;
     uint32_t nr = 0;
     const uint32_t edst = (uint32_t)wave * 8192u;   // this wavefront's eighth of a fill, in memory and in LDS
-    // fill 0 of a column tile -> buffer 0: eight loads of 1 KiB, memory straight into LDS
-    auto load_first_fill = [&](const int ct) __attribute__((always_inline)) {
-        const uint32_t eoff = (uint32_t)(ct * F) * (uint32_t)kPxFillBytes + edst;
+    // the first fill of a tile (column tile incl. K split ctv) -> buffer 0: eight loads of 1 KiB, memory straight
+    // into LDS
+    auto load_first_fill = [&](const int ctv) __attribute__((always_inline)) {
+        const int ksi = ctv / p.plan.n_col_tiles;
+        const uint32_t eoff = (uint32_t)((ctv - ksi * p.plan.n_col_tiles) * F + ksi * Fs) * (uint32_t)kPxFillBytes + edst;
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -164,14 +168,21 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
         load_first_fill(ct0);
     }
     for (int tile = tile_first; tile < tile_end; tile += tile_step) {
-        int rt, ct;
-        decode(tile, rt, ct);
-        int ct_next = ct;
+        int rt, ctv;
+        decode(tile, rt, ctv);
+        int ctv_next = ctv;
         const bool has_next = tile + tile_step < tile_end;
         if (has_next) {
             int rt_next;
-            decode(tile + tile_step, rt_next, ct_next);
+            decode(tile + tile_step, rt_next, ctv_next);
         }
+        const int ksi = ctv / p.plan.n_col_tiles;           // K split of this tile
+        const int ct = ctv - ksi * p.plan.n_col_tiles;
+        const int f0 = ksi * Fs;                            // its fills: [f0, f0 + Ft)
+        const int Ft = F - f0 < Fs ? F - f0 : Fs;
+        const int ksi_next = ctv_next / p.plan.n_col_tiles;
+        const uint32_t first_fill = (uint32_t)(ct * F + f0);
+        const uint32_t first_fill_next = (uint32_t)((ctv_next - ksi_next * p.plan.n_col_tiles) * F + ksi_next * Fs);
         const TileRows t = tile_rows_of<R, true>(p, rt, wave);
         if (rt != prev_rt) {
             prev_rt = rt;
@@ -180,23 +191,29 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
         const uint32_t nr_s = __builtin_amdgcn_readfirstlane(nr);
 
         // ---- activation cursor: (tap, quad pair) of the fill whose activations are fetched next ----
-        int cur_fill = 0, cur_qp = 0, cur_kh = 0, cur_kw = 0;
+        int cur_fill = 0, cur_qp = 0, cur_kh = 0, cur_kw = 0;   // cur_fill counts from the tile's first fill
+        if (f0) {
+            const int tap = f0 / qpairs;
+            cur_qp = f0 - tap * qpairs;
+            cur_kh = tap / g.KW;
+            cur_kw = tap - cur_kh * g.KW;
+        }
         uint32_t idx_tap[R];
-        tap_offsets<R>(p, park, 0, 0, zp_row, idx_tap);
+        tap_offsets<R>(p, park, cur_kh, cur_kw, zp_row, idx_tap);
         auto advance_cursor = [&]() __attribute__((always_inline)) {
             ++cur_fill;
             if (++cur_qp == qpairs) {
                 cur_qp = 0;
                 if (++cur_kw == g.KW) { cur_kw = 0; ++cur_kh; }
-                if (cur_fill < F)   // pixel 0's activations are fetched whether the wavefront has a pixel or not
+                if (cur_fill < Ft)   // pixel 0's activations are fetched whether the wavefront has a pixel or not
                     tap_offsets<R>(p, park, cur_kh, cur_kw, zp_row, idx_tap, nr_s > 1u ? nr_s : 1u);
             }
         };
         uint32_t fA[R], sA[R], fB[R], sB[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            fA[r] = ld_u32(xq_rsrc, idx_tap[r] + dlf, 0);
-            sA[r] = ld_u32(xq_rsrc, idx_tap[r] + dls, 0);
+            fA[r] = ld_u32(xq_rsrc, idx_tap[r] + dlf, (uint32_t)cur_qp * 2u * quad_bytes);
+            sA[r] = ld_u32(xq_rsrc, idx_tap[r] + dls, (uint32_t)cur_qp * 2u * quad_bytes);
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of fill 0 and its activations are there
         __syncthreads();                      // ... and everyone's; the previous tile's epilogue is done with LDS
@@ -208,7 +225,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
             for (int j = 0; j < NT; ++j)
                 acc[r][j] = 0;
 
-        if (F > 1)
+        if (Ft > 1)
             advance_cursor();   // entering phase p the cursor stands on fill p + 1
         auto phase = [&](const int pcur, uint32_t (&f_cur)[R], uint32_t (&s_cur)[R], uint32_t (&f_next)[R],
                          uint32_t (&s_next)[R], auto buf_tag) __attribute__((always_inline)) {
@@ -216,9 +233,9 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
             // What lands in the other buffer during this phase: the next fill of this tile.  Behind the last fill of
             // an even count the other buffer is buffer 0, and it gets the first fill of the workgroup's next tile;
             // otherwise the last fill once more (never used).
-            uint32_t fill_next = (uint32_t)(ct * F + pcur + 1);
-            if (pcur + 1 >= F)
-                fill_next = (BUF == 1 && has_next) ? (uint32_t)(ct_next * F) : (uint32_t)(ct * F + F - 1);
+            uint32_t fill_next = first_fill + (uint32_t)(pcur + 1);
+            if (pcur + 1 >= Ft)
+                fill_next = (BUF == 1 && has_next) ? first_fill_next : first_fill + (uint32_t)(Ft - 1);
             const uint32_t eoff = fill_next * (uint32_t)kPxFillBytes + edst;
             const uint32_t qoff = (uint32_t)cur_qp * 2u * quad_bytes;
             uint32_t stmp;
@@ -231,21 +248,21 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
                             __builtin_amdgcn_readfirstlane(edst), __builtin_amdgcn_readfirstlane(eoff), e_rsrc, xq_rsrc,
                             __builtin_amdgcn_readfirstlane(qoff));
             (void)stmp;
-            if (pcur + 2 < F)
+            if (pcur + 2 < Ft)
                 advance_cursor();
             __syncthreads();
         };
-        for (int pcur = 0; pcur < F; pcur += 2) {
+        for (int pcur = 0; pcur < Ft; pcur += 2) {
             phase(pcur, fA, sA, fB, sB, std::integral_constant<int, 0>());
-            if (pcur + 1 < F)
+            if (pcur + 1 < Ft)
                 phase(pcur + 1, fB, sB, fA, sA, std::integral_constant<int, 1>());
         }
         // An odd count of fills ends on buffer 0, which every wavefront has now left: the next tile's first fill
         // goes there while the epilogue runs.  The epilogue turns its outputs through buffer 1 either way.
-        if ((F & 1) && has_next)
-            load_first_fill(ct_next);
+        if ((Ft & 1) && has_next)
+            load_first_fill(ctv_next);
         fix_even_columns<R, NT>(acc);
-        store_tile<NT, OUT_I32>(p, acc, t, ct, 0, nr_s, lane, wave, lds_px + kPxFillBytes);
+        store_tile<NT, OUT_I32>(p, acc, t, ct, ksi, nr_s, lane, wave, lds_px + kPxFillBytes);
     }
 }
 
@@ -265,7 +282,9 @@ static hipError_t launch_px_one(const DenseParams &p, hipStream_t stream)
 
 hipError_t launch_dense_px(const DenseParams &p, bool out_i32, hipStream_t stream)
 {
-    if (p.plan.nt != 16 || p.plan.k_splits != 1 || (p.plan.fills & 1) || (p.g.C4 & 1) || !p.px_rows)
+    if (p.plan.nt != 16 || (p.plan.fills & 1) || (p.g.C4 & 1) || !p.px_rows)
+        return hipErrorInvalidValue;
+    if (p.plan.k_splits > 1 && ((p.plan.fills_per_split & 1) || !out_i32))   // a split covers whole pre-expanded fills
         return hipErrorInvalidValue;
     return out_i32 ? launch_px_one<true>(p, stream) : launch_px_one<false>(p, stream);
 }
