@@ -290,12 +290,19 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
         // thread -> (pixel column, channel quad) once; then it walks down the rows and across the columns, sixteen
         // 16-byte loads in flight at a time.  The loads are unconditional (coordinates clamped into the image, the
         // result replaced by zeros afterwards) so that each store waits for its own load only.
+        // A narrow image leaves most threads without a column: they then take further rows (rpar rows side by side).
         constexpr int kInFlight = 16;
-        const int q = t % g.C4, w0 = t / g.C4, wstep = nthreads / g.C4;
-        const int wsteps = (g.W + wstep - 1) / wstep;
-        const int iters = in_rows * wsteps;
+        const int q = t % g.C4, wstep = nthreads / g.C4;
+        const int rpar = wstep >= 2 * g.W ? wstep / g.W : 1;
+        int w0 = t / g.C4, r0 = 0;
+        if (rpar > 1) {
+            r0 = w0 / g.W;
+            w0 = r0 < rpar ? w0 - r0 * g.W : g.W;   // threads beyond the last whole row: no column
+        }
+        const int wsteps = rpar > 1 ? 1 : (g.W + wstep - 1) / wstep;
+        const int iters = ((in_rows + rpar - 1) / rpar) * wsteps;
         const float *const xn = x + (int64_t)n * g.H * g.W * g.C + q * 4;
-        int r_next = 0, ws_next = 0; // (row, column step) of the next item
+        int r_next = r0, ws_next = 0; // (row, column step) of the next item
         for (int it0 = 0; it0 < iters; it0 += kInFlight) {
             float4 v[kInFlight];
             int rr[kInFlight], ww[kInFlight];
@@ -305,12 +312,14 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
                 ww[u] = w0 + ws_next * wstep;
                 if (++ws_next == wsteps) {
                     ws_next = 0;
-                    ++r_next;
+                    r_next += rpar;
                 }
                 int ih = ih_first + rr[u];
                 ih = ih < 0 ? 0 : (ih >= g.H ? g.H - 1 : ih);
                 const int wc = ww[u] < g.W ? ww[u] : g.W - 1;
-                v[u] = *reinterpret_cast<const float4 *>(xn + ((int64_t)ih * g.W + wc) * g.C);
+                v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (it0 + u < iters)   // the same for the whole workgroup: no load for items nobody has
+                    v[u] = *reinterpret_cast<const float4 *>(xn + ((int64_t)ih * g.W + wc) * g.C);
             }
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u) {
@@ -319,7 +328,7 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
                 float4 f = fake_quant_value4(v[u], qt);
                 if (!in_image)
                     f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);   // rows outside the image are zeros
-                if (it0 + u < iters && ww[u] < g.W) {
+                if (it0 + u < iters && rr[u] < in_rows && ww[u] < g.W) {
                     *reinterpret_cast<float4 *>(&rows[(rr[u] * g.W + ww[u]) * pitch + q * 4]) = f;
                     if (xq && in_image && ih >= own_lo && ih < own_hi)
                         xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + ww[u]] =
