@@ -139,8 +139,10 @@ int axc_qint32_range_for_multiplication(float min_a, float max_a, float min_b, f
 
 /* How the dense kernel would cut this layer on the current device (for tools and tests; the reference has no
  * counterpart, its launch shapes are fixed in cuda/approx_nn_conv_kernels.cu:296-627):
- * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups }. */
-int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6]);
+ * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups,
+ *          fills of 64 filter entries per K split, 1 if the layer runs out of pre-expanded rows (given a workspace of
+ *          the size axc_conv2d_workspace_bytes reports) else 0 }. */
+int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[8]);
 /* Pins the tile width the planner uses (16, 32 or 64 columns; 0 = its own choice, the default), process-wide, for
  * tests and timing of the wider-tile kernel variants.  The environment variable AXC_TILE_COLUMNS gives the initial
  * value and is read once, when the library is loaded.  Like axc_set_preexpand it is process-wide; a workspace query and

@@ -135,6 +135,49 @@ def test_attr_errors_mirror_the_reference(ops, lib):
     assert rc == 1 and msg == "ApproxConv2DOp: Patch too large for buffer"
 
 
+def test_tile_plans_fit_the_kernels(ops, lib):
+    """What the planner hands the LUT-GEMM kernels, over many layers and all pinned modes (the query needs no GPU:
+    without one it plans for 256 CUs).  A tile holds at most 8 wavefronts x 2 * 64 / columns pixel slots of 64 pixels,
+    the row tiles cover the pixels without an empty one, every K split has fills, and pre-expanded rows only come with
+    16-column tiles, channel quads in pairs and splits of whole pairs of fills."""
+    shapes = []
+    for n, hw in [(1, 1), (1, 7), (2, 8), (4, 14), (64, 14), (64, 28), (16, 56), (64, 56), (128, 32), (128, 8), (3, 33)]:
+        for c, co in [(3, 16), (8, 16), (16, 16), (64, 64), (40, 20), (256, 1024), (512, 128), (128, 130), (2048, 512)]:
+            for k in (1, 3):
+                if n * hw * hw * max(c, co) <= 64 * 56 * 56 * 1024 and k * k * c < 32768:
+                    shapes.append(((n, hw, hw, c), (k, k, c, co)))
+    seen_px = seen_split = seen_px_split = 0
+    try:
+        for columns, mode in [(0, 0), (0, 1), (0, -1), (16, 1), (32, 0), (64, 0)]:
+            assert lib.axc_set_tile_columns(columns) == 0 and lib.axc_set_preexpand(mode) == 0
+            for xs, fs in shapes:
+                pl = ops.conv2d_tile_plan(xs, fs)
+                nt, rows, ks = pl["columns_per_tile"], pl["rows_per_tile"], pl["k_splits"]
+                m = xs[0] * xs[1] * xs[2]
+                what = (columns, mode, xs, fs, pl)
+                assert nt in (16, 32, 64) and (columns == 0 or nt == columns), what
+                assert rows % 64 == 0 and 0 < rows // 64 <= 8 * 2 * (64 // nt), what
+                assert (pl["row_tiles"] - 1) * rows < m <= pl["row_tiles"] * rows, what
+                assert pl["column_tiles"] == -(-fs[3] // nt), what
+                tiles = pl["row_tiles"] * pl["column_tiles"] * ks
+                assert 1 <= pl["workgroups"] <= tiles, what
+                fps = pl["fills_per_split"]
+                if xs[3] % 4 == 0:   # (other channel counts may use the flat layout, which counts quads per filter row)
+                    fills = fs[0] * fs[1] * (xs[3] // 4) * (nt // 16)
+                    assert 1 <= ks <= 16 and (ks - 1) * fps < fills <= ks * fps, what
+                if pl["preexpanded_rows"]:
+                    assert mode >= 0 and nt == 16 and fps % 2 == 0 and (xs[3] % 4 or (xs[3] // 4) % 2 == 0), what
+                    assert pl["column_tiles"] * (fps * ks // 2) * 65536 <= (192 << 20) + ks * 65536, what
+                elif mode == 1 and nt == 16 and xs[3] % 8 == 0:
+                    assert pl["column_tiles"] * fs[0] * fs[1] * (xs[3] // 8) * 65536 > 192 << 20, what
+                seen_px += pl["preexpanded_rows"]
+                seen_split += ks > 1
+                seen_px_split += pl["preexpanded_rows"] and ks > 1
+    finally:
+        assert lib.axc_set_tile_columns(0) == 0 and lib.axc_set_preexpand(0) == 0
+    assert seen_px > 50 and seen_split > 50 and seen_px_split > 5
+
+
 def test_workspace_sizes(ops, lib):
     desc = ops.make_desc((64, 56, 56, 64), (3, 3, 64, 64), (1, 1, 1, 1), "SAME")
     rc, n = _ws(lib, desc)

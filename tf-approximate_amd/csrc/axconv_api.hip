@@ -1156,7 +1156,7 @@ int axc_qint32_range_for_multiplication(float min_a, float max_a, float min_b, f
     return AXC_OK;
 }
 
-int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6])
+int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[8])
 {
     if (!plan)
         return fail(AXC_INVALID_ARGUMENT, "null argument");
@@ -1170,6 +1170,8 @@ int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[6])
     plan[3] = pd.plan.n_col_tiles;
     plan[4] = pd.plan.k_splits;
     plan[5] = pd.plan.grid;
+    plan[6] = pd.plan.k_splits > 1 ? pd.plan.fills_per_split : pd.plan.fills;
+    plan[7] = pd.plan.px;
     return AXC_OK;
 }
 

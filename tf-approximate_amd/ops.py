@@ -323,9 +323,10 @@ def conv2d_tile_plan(input_shape, filter_shape, strides=(1, 1, 1, 1), padding="S
     """The dense kernel's tile plan for a layer on the current device, as a dict."""
     lib = _lib.load()
     desc = make_desc(tuple(input_shape), tuple(filter_shape), list(strides), padding, (), "NHWC", list(dilations), 8)
-    plan = (ctypes.c_int32 * 6)()
+    plan = (ctypes.c_int32 * 8)()
     _check(lib.axc_conv2d_tile_plan(ctypes.byref(desc), plan))
-    keys = ("columns_per_tile", "rows_per_tile", "row_tiles", "column_tiles", "k_splits", "workgroups")
+    keys = ("columns_per_tile", "rows_per_tile", "row_tiles", "column_tiles", "k_splits", "workgroups",
+            "fills_per_split", "preexpanded_rows")
     return dict(zip(keys, [int(v) for v in plan]))
 
 
