@@ -760,7 +760,14 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         const DensePlan &pl = pd.plan;
         const int64_t tiles = (int64_t)pl.n_row_tiles * pl.n_col_tiles * pl.k_splits;
         p.stagger_sleeps = 0;
-        if (pl.k_splits == 1 && pl.fills <= 16 && tiles >= (int64_t)8 * pl.grid) {
+        p.stagger_groups = 2;
+        if (use_px && pl.k_splits == 1 && tiles >= (int64_t)2 * pl.grid) {
+            // Out of pre-expanded rows, with any K and from two tiles per workgroup on: four groups, each one sleep
+            // period (~8 000 cycles, about what a tile's output stores take) behind the one before it (measured:
+            // 1x1 64->256 @56x56 -8 %, 128->512 @28x28 -3 %, the other multi-tile layers -0.5 to -2 %).
+            p.stagger_sleeps = 1;
+            p.stagger_groups = 4;
+        } else if (pl.k_splits == 1 && pl.fills <= 16 && tiles >= (int64_t)8 * pl.grid) {
             const double per_simd = (double)((pl.rows_per_tile / 64 + 3) / 4);
             const double tile_cycles = (double)pl.fills * (1700.0 + per_simd * 290.0) + 6000.0; // the planner's model
             const int sleeps = (int)(0.45 * tile_cycles / 8128.0 + 0.5);

@@ -101,7 +101,8 @@ struct DenseParams {
     const LayerQuant *lq_dev;    // not null: epilogue constants come from here instead of the four floats above
     const float *bias;           // not null: added to every output column after the epilogue
     int relu;                    // 1: max(x, 0) last
-    int stagger_sleeps;          // s_sleep(127) periods by which every second group of workgroups starts late (0: none)
+    int stagger_sleeps;          // s_sleep(127) periods by which group g of the workgroups starts late, times g (0: none)
+    int stagger_groups;          // g = 0 .. stagger_groups - 1 in turn (2: every second group, the only form lutgemm_expand has)
     const uint16_t *px_rows;     // pre-expanded rows [n_col_tiles][fills / 2][256][128] (lutgemm_px_kernel only)
     uint32_t px_bytes;
     // Addressing of xq.  Usual layout: dwords of four channels, [N][H][C4][W].  Flat layout (channel counts that are

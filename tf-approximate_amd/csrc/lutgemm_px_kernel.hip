@@ -144,9 +144,11 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_px_kernel(const DensePa
         tile_end = ntiles;
         tile_step = G;
     }
-    if (p.stagger_sleeps && ((tile_first / (n_col < kPxBlockCols ? n_col : kPxBlockCols)) & 1))
-        for (int i = 0; i < p.stagger_sleeps; ++i)
+    if (p.stagger_sleeps) {
+        const int late = p.stagger_sleeps * ((tile_first / (n_col < kPxBlockCols ? n_col : kPxBlockCols)) % p.stagger_groups);
+        for (int i = 0; i < late; ++i)
             __builtin_amdgcn_s_sleep(127);
+    }
 
     int prev_rt = -1;
     uint32_t nr = 0;
