@@ -258,8 +258,12 @@ __device__ __forceinline__ void filter_pack_element(const int64_t i, const float
 // Pixels are padded to C + 4 floats so that the 16-byte reads of neighbouring threads fall into different banks.
 // bid / nblocks: index of this workgroup among those that do this work (in dispatch order, so that bid & 7 is
 // the XCD); nthreads: the threads of the workgroup that take part (the others only meet the barrier).
+// wseg: output columns per workgroup.  wseg == OW: whole rows.  Less (wide rows of many channels, which would not
+// fit LDS otherwise): a band is cut into column segments, each with the input columns under it in LDS (SEG; without
+// it the code is the one for whole rows, with no trace of the segments).
+template <bool SEG>
 __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x, const ConvGeom &g, const int rb,
-                                                     const int in_rows, const TensorQuant &tq,
+                                                     const int in_rows, const int wseg, const TensorQuant &tq,
                                                      const LayerQuant *__restrict__ lq_dev, float *__restrict__ psum,
                                                      uint32_t *__restrict__ xq, const int bid_in, const int nblocks,
                                                      const int nthreads, const FilterWork &fw)
@@ -278,11 +282,26 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
     // consecutive bands (which share input rows) go to the same XCD: blocks are dealt round-robin over 8 XCDs
     const int per_xcd = nblocks / 8, extra = nblocks % 8, xcd = bid_in & 7;
     const int bid = xcd * per_xcd + (xcd < extra ? xcd : extra) + (bid_in >> 3);
-    const int n = bid / bands;
-    const int oh0 = (bid - n * bands) * rb;
+    const int segs = SEG ? (g.OW + wseg - 1) / wseg : 1;
+    const int nb = SEG ? bid / segs : bid, seg = SEG ? bid - nb * segs : 0;   // nb: (image, band)
+    const int n = nb / bands, band = nb - n * bands;
+    const int oh0 = band * rb;
     const int ih_first = oh0 * g.sh - g.ph;  // input row held in LDS row 0 (may lie outside the image)
     const int own_lo = oh0 * g.sh;           // owned input rows: [own_lo, own_hi)
     const int own_hi = (oh0 + rb >= g.OH) ? g.H : (oh0 + rb) * g.sh;
+    const int ow0 = SEG ? seg * wseg : 0, ow1 = (SEG && ow0 + wseg < g.OW) ? ow0 + wseg : g.OW;   // output columns [ow0, ow1)
+    const int segw = ow1 - ow0;
+    // input columns [iw_lo, iw_lo + wc) are held in LDS; [own_clo, own_chi) of them are this workgroup's to quantize
+    int iw_lo = 0, wc = g.W, own_clo = 0, own_chi = g.W;
+    if (SEG) {
+        iw_lo = ow0 * g.sw - g.pw;
+        iw_lo = iw_lo < 0 ? 0 : iw_lo;
+        int iw_hi = (ow1 - 1) * g.sw - g.pw + (g.KW - 1) * g.dw + 1;
+        iw_hi = iw_hi > g.W ? g.W : iw_hi;
+        wc = iw_hi - iw_lo;
+        own_clo = ow0 * g.sw;
+        own_chi = ow1 == g.OW ? g.W : ow1 * g.sw;
+    }
     const int pitch = g.C + 4;
     if (t >= nthreads) {
         // not taking part in the copy
@@ -293,13 +312,13 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
         // A narrow image leaves most threads without a column: they then take further rows (rpar rows side by side).
         constexpr int kInFlight = 16;
         const int q = t % g.C4, wstep = nthreads / g.C4;
-        const int rpar = wstep >= 2 * g.W ? wstep / g.W : 1;
+        const int rpar = wstep >= 2 * wc ? wstep / wc : 1;
         int w0 = t / g.C4, r0 = 0;
         if (rpar > 1) {
-            r0 = w0 / g.W;
-            w0 = r0 < rpar ? w0 - r0 * g.W : g.W;   // threads beyond the last whole row: no column
+            r0 = w0 / wc;
+            w0 = r0 < rpar ? w0 - r0 * wc : wc;   // threads beyond the last whole row: no column
         }
-        const int wsteps = rpar > 1 ? 1 : (g.W + wstep - 1) / wstep;
+        const int wsteps = rpar > 1 ? 1 : (wc + wstep - 1) / wstep;
         const int iters = ((in_rows + rpar - 1) / rpar) * wsteps;
         const float *const xn = x + (int64_t)n * g.H * g.W * g.C + q * 4;
         int r_next = r0, ws_next = 0; // (row, column step) of the next item
@@ -316,10 +335,10 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
                 }
                 int ih = ih_first + rr[u];
                 ih = ih < 0 ? 0 : (ih >= g.H ? g.H - 1 : ih);
-                const int wc = ww[u] < g.W ? ww[u] : g.W - 1;
+                const int wcl = iw_lo + (ww[u] < wc ? ww[u] : wc - 1);
                 v[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                 if (it0 + u < iters)   // the same for the whole workgroup: no load for items nobody has
-                    v[u] = *reinterpret_cast<const float4 *>(xn + ((int64_t)ih * g.W + wc) * g.C);
+                    v[u] = *reinterpret_cast<const float4 *>(xn + ((int64_t)ih * g.W + wcl) * g.C);
             }
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u) {
@@ -328,10 +347,11 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
                 float4 f = fake_quant_value4(v[u], qt);
                 if (!in_image)
                     f = make_float4(0.0f, 0.0f, 0.0f, 0.0f);   // rows outside the image are zeros
-                if (it0 + u < iters && rr[u] < in_rows && ww[u] < g.W) {
-                    *reinterpret_cast<float4 *>(&rows[(rr[u] * g.W + ww[u]) * pitch + q * 4]) = f;
-                    if (xq && in_image && ih >= own_lo && ih < own_hi)
-                        xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + ww[u]] =
+                if (it0 + u < iters && rr[u] < in_rows && ww[u] < wc) {
+                    *reinterpret_cast<float4 *>(&rows[(rr[u] * wc + ww[u]) * pitch + q * 4]) = f;
+                    const int iw = iw_lo + ww[u];
+                    if (xq && in_image && ih >= own_lo && ih < own_hi && (!SEG || (iw >= own_clo && iw < own_chi)))
+                        xq[(((int64_t)n * g.H + ih) * g.C4 + q) * g.W + iw] =
                             phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
                             (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
                             (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
@@ -340,7 +360,7 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
             }
         }
     } else {
-        const int quads_per_row = g.W * g.C4;
+        const int quads_per_row = wc * g.C4;
         const int total = in_rows * quads_per_row;
         for (int i = t; i < total; i += nthreads) {
             const int r = i / quads_per_row, rem = i - r * quads_per_row;
@@ -349,11 +369,11 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
             float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if ((unsigned)ih < (unsigned)g.H)
                 v = fake_quant_value4(
-                    *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + w) * g.C + q * 4), qt);
-            *reinterpret_cast<float4 *>(&rows[(r * g.W + w) * pitch + q * 4]) = v;
+                    *reinterpret_cast<const float4 *>(x + (((int64_t)n * g.H + ih) * g.W + iw_lo + w) * g.C + q * 4), qt);
+            *reinterpret_cast<float4 *>(&rows[(r * wc + w) * pitch + q * 4]) = v;
         }
     }
-    float *const zero_px = rows + (size_t)in_rows * g.W * pitch; // one pixel of zeros behind the rows (see below)
+    float *const zero_px = rows + (size_t)in_rows * wc * pitch; // one pixel of zeros behind the rows (see below)
     if (t < g.C4)
         *reinterpret_cast<float4 *>(zero_px + t * 4) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     __syncthreads();
@@ -361,13 +381,13 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
     // CU (wavefronts of a block are spread over the SIMDs in order), so that their chains do not share a SIMD.
     const int rot = ((bid_in >> 8) + (bid_in >> 3)) & 3;
     const int tc = (t + (int)blockDim.x - rot * 64) % (int)blockDim.x;
-    const int ohl = tc / g.OW, ow = tc - ohl * g.OW;
+    const int ohl = tc / segw, ow = ow0 + tc - ohl * segw;
     const int oh = oh0 + ohl;
     if (ohl >= rb) {
         // No chain for this thread.  If the launch asks for it, it packs filter codes meanwhile - but only from
         // wavefronts that share no SIMD with a chain (wavefront w of the block sits on SIMD w mod 4): a chain
         // runs as fast as its wavefront gets to issue, and any other work on its SIMD takes issue slots from it.
-        const int chain_waves = (rb * g.OW + 63) / 64;
+        const int chain_waves = (rb * segw + 63) / 64;
         const int wave = tc >> 6; // counted from the first chain wavefront
         if (fw.pack_total > 0 && (wave & 3) >= chain_waves) {
             const int waves = (int)blockDim.x >> 6;
@@ -399,7 +419,7 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
         auto tap_src = [&]() -> const float4 * {
             const int iw = iw0 + kw * g.dw;
             const bool ok = kh < g.KH && (unsigned)iw < (unsigned)g.W;
-            return reinterpret_cast<const float4 *>(ok ? rows + ((ohl * g.sh + kh * g.dh) * g.W + iw) * pitch : zero_px);
+            return reinterpret_cast<const float4 *>(ok ? rows + ((ohl * g.sh + kh * g.dh) * wc + iw - iw_lo) * pitch : zero_px);
         };
         const float4 *src = tap_src();
         auto read = [&](float4(&w)[kBatch]) {
@@ -450,7 +470,7 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
             const int iw = iw0 + kw * g.dw;
             if ((unsigned)iw >= (unsigned)g.W)
                 continue;
-            const float *src = &rows[(r * g.W + iw) * pitch];
+            const float *src = &rows[(r * wc + iw - iw_lo) * pitch];
 #pragma unroll 8
             for (int q = 0; q < g.C4; ++q) {
                 const float4 v = *reinterpret_cast<const float4 *>(src + q * 4);
@@ -964,7 +984,7 @@ __device__ __forceinline__ void patch_sums_deep_body(const float *__restrict__ x
 }
 
 __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, const ConvGeom g, int rb,
-                                                                int in_rows, int nthreads, const TensorQuant tq,
+                                                                int in_rows, int nthreads, int wseg, const TensorQuant tq,
                                                                 const LayerQuant *__restrict__ lq_dev,
                                                                 float *__restrict__ psum, uint32_t *__restrict__ xq,
                                                                 const FilterWork fw)
@@ -995,8 +1015,12 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
         patch_sums_flat_body(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8, in_rows);
         return;
     }
-    patch_sums_rows_body(x, g, rb, in_rows, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
-                         (int)gridDim.x - fw.blocks8, nthreads, fw);
+    if (wseg >= g.OW)
+        patch_sums_rows_body<false>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
+                                    (int)gridDim.x - fw.blocks8, nthreads, fw);
+    else
+        patch_sums_rows_body<true>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
+                                   (int)gridDim.x - fw.blocks8, nthreads, fw);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -1355,23 +1379,40 @@ hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const Ten
 // such wavefronts interleaves them at no better than one add per ~1.9 ns, so lanes left idle by a thin band and
 // chain wavefronts that share a SIMD are what make deep layers slow.  Blocks beyond what the CUs hold at once
 // run as further rounds; the blocks that sum filter columns in the same launch (sum_blocks) count like the others.
-static void choose_band(const ConvGeom &g, int64_t row_bytes, int sum_blocks, int *rb_out, int *in_rows_out)
+// Rows of many channels fit LDS only a few at a time, or not at all: the band is then cut into column segments of
+// wseg output columns, each workgroup holding only the input columns under its segment (input_columns_under).
+// Measured on the layers of the networks: where whole rows leave room for one workgroup per CU only, segments that
+// let two be resident (the copy of one runs under the chains of the other) are 10-20 % faster, the more pixels per
+// workgroup the better; with room for two, whole rows stay ahead.
+static int input_columns_under(const ConvGeom &g, int wseg)
+{
+    if (wseg >= g.OW)
+        return g.W;
+    const int cols = (wseg - 1) * g.sw + (g.KW - 1) * g.dw + 1;
+    return cols < g.W ? cols : g.W;
+}
+
+// Least estimated time over the band heights of one segment width; returns false if no band fits.
+static bool best_band(const ConvGeom &g, int wseg, int sum_blocks, int64_t lds_limit, int *rb_out, int *in_rows_out,
+                      double *t_out, int64_t *lds_out)
 {
     const int cus = device_cus();
     const double K = (double)g.KH * g.KW * g.C;
     const int64_t lds_max = 160 * 1024;
-    double best = 0.0;
-    for (int cand = 1; cand <= g.OH && cand * g.OW <= 1024; ++cand) {
+    const int nsegs = (g.OW + wseg - 1) / wseg;
+    const int64_t row_bytes = (int64_t)input_columns_under(g, wseg) * (g.C + 4) * 4;
+    bool found = false;
+    for (int cand = 1; cand <= g.OH && cand * wseg <= 1024; ++cand) {
         const int rows_needed = (cand - 1) * g.sh + (g.KH - 1) * g.dh + 1;
         const int64_t lds = rows_needed * row_bytes + (int64_t)(g.C + 4) * 4;
-        if (lds > lds_max)
+        if (lds > lds_limit)
             break;
-        const int chains = cand * g.OW;
+        const int chains = cand * wseg;
         const int block_threads = chains <= 512 ? 512 : 1024;
         int64_t per_cu = lds_max / lds;
         if (per_cu > 2048 / block_threads)
             per_cu = 2048 / block_threads;
-        const int64_t blocks = (int64_t)g.N * ((g.OH + cand - 1) / cand) + sum_blocks; // all of one LDS size
+        const int64_t blocks = (int64_t)g.N * ((g.OH + cand - 1) / cand) * nsegs + sum_blocks; // all of one LDS size
         const int64_t rounds = (blocks + cus * per_cu - 1) / (cus * per_cu);
         int64_t resident = (blocks + cus - 1) / cus;
         if (resident > per_cu)
@@ -1380,10 +1421,72 @@ static void choose_band(const ConvGeom &g, int64_t row_bytes, int sum_blocks, in
         const double copy_ns = (double)(resident * lds) / 17.0;
         const double chain_ns = K * 2.75 * (double)((chain_waves + 3) / 4);
         const double t = (double)rounds * (copy_ns + chain_ns);
-        if (cand == 1 || t < best) {
-            best = t;
+        if (!found || t < *t_out) {
+            found = true;
+            *t_out = t;
             *rb_out = cand;
             *in_rows_out = rows_needed;
+            *lds_out = lds;
+        }
+    }
+    return found;
+}
+
+static void choose_band(const ConvGeom &g, int sum_blocks, int *rb_out, int *in_rows_out, int *wseg_out)
+{
+    const int64_t lds_max = 160 * 1024, lds_two = lds_max / 2;
+    double t = 0.0;
+    int64_t lds = 0;
+    *rb_out = 0;
+    *wseg_out = g.OW;
+    const bool whole = best_band(g, g.OW, sum_blocks, lds_max, rb_out, in_rows_out, &t, &lds);
+    // whole rows with room for two workgroups per CU, or with no more workgroups than CUs: nothing to gain
+    if (whole && (lds <= lds_two || (int64_t)g.N * ((g.OH + *rb_out - 1) / *rb_out) + sum_blocks <= device_cus()))
+        return;
+    // segments with room for two workgroups per CU: the most pixels per workgroup, at least eight, and more
+    // segments only for 15 % more pixels (thin segments copy more halo and fill their wavefronts worse).  Not under
+    // long chains (K above ~3000: 8 us and more), where the largest workgroup that fits is the better one.
+    int best_chains = 7, last_wseg = g.OW;
+    const bool long_chains = (int64_t)g.KH * g.KW * g.C > 3000;
+    for (int segs : {2, 3, 4, 6, 8}) {
+        if (long_chains)
+            break;
+        const int wseg = (g.OW + segs - 1) / segs;
+        if (wseg == last_wseg || wseg < 4)
+            continue;
+        last_wseg = wseg;
+        const int64_t row_bytes = (int64_t)input_columns_under(g, wseg) * (g.C + 4) * 4;
+        for (int cand = 1; cand <= g.OH && cand * wseg <= 1024; ++cand) {
+            const int rows_needed = (cand - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+            if (rows_needed * row_bytes + (int64_t)(g.C + 4) * 4 > lds_two)
+                break;
+            if (cand * wseg > best_chains && (best_chains == 7 || cand * wseg * 100 > best_chains * 115 ||
+                                              wseg == *wseg_out)) {
+                best_chains = cand * wseg;
+                *rb_out = cand;
+                *in_rows_out = rows_needed;
+                *wseg_out = wseg;
+            }
+        }
+    }
+    if (best_chains > 7 || whole)
+        return;
+    // whole rows do not fit and neither does a pair of segments: one workgroup per CU, by the estimate
+    last_wseg = g.OW;
+    bool any = false;
+    for (int segs : {2, 3, 4, 6, 8}) {
+        const int wseg = (g.OW + segs - 1) / segs;
+        if (wseg == last_wseg || wseg < 4)
+            continue;
+        last_wseg = wseg;
+        int rb = 0, in_rows = 0;
+        double ts = 0.0;
+        if (best_band(g, wseg, sum_blocks, lds_max, &rb, &in_rows, &ts, &lds) && (!any || ts < t)) {
+            any = true;
+            t = ts;
+            *rb_out = rb;
+            *in_rows_out = in_rows;
+            *wseg_out = wseg;
         }
     }
 }
@@ -1416,9 +1519,10 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
         // 1x1, stride 1, no padding, and a band would hold few pixels (many channels): the flat-list variant
         const bool flat = g.KH == 1 && g.KW == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 &&
                           rb * g.OW < 192;
-        if (!flat && rb > 0)
-            choose_band(g, row_bytes, (filter_job && filter_job->fsum && filter_job->filter) ? (int)blocks_for(g.Co, kFsCols) : 0,
-                        &rb, &in_rows);
+        int wseg = g.OW;   // output columns per workgroup: whole rows unless choose_band cuts them
+        if (!flat)
+            choose_band(g, (filter_job && filter_job->fsum && filter_job->filter) ? (int)blocks_for(g.Co, kFsCols) : 0,
+                        &rb, &in_rows, &wseg);
         // ... and with many channels and too few pixels to give every CU a workgroup of 64, the variant built around
         // the chain of adds
         const bool deep = flat && g.C >= 512 && g.M < (int64_t)64 * device_cus();
@@ -1431,21 +1535,28 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
             in_rows = g.M >= (int64_t)2 * 16 * device_cus() ? 16 : 8;
         }
         if (rb > 0 || flat) {
-            int threads = ((rb * g.OW + 63) / 64) * 64;
+            int threads = ((rb * wseg + 63) / 64) * 64;
             threads = threads < 512 ? 512 : threads;   // the copy into LDS wants more threads than there are pixels
             // Band b owns input rows [b*rb*sh, (b+1)*rb*sh), the last band up to H.  They are quantized by the
             // block that holds them if every band's window (rows b*rb*sh - ph onwards, in_rows of them) contains
-            // its owned rows, the last window reaches the last image row, and the fast copy loop is in use.
+            // its owned rows, the last window reaches the last image row, and the fast copy loop is in use.  The
+            // same along the row where a band is cut into column segments (segment s owns input columns
+            // [s*wseg*sw, (s+1)*wseg*sw), the last one up to W).
+            const bool segmented = !flat && wseg < g.OW;
             const bool fuse = xq_fused && fused &&
                               (flat || (g.sh - 1 + g.ph <= (g.KH - 1) * g.dh &&
-                                        (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0));
+                                        (g.OH - 1) * g.sh - g.ph + (g.KH - 1) * g.dh >= g.H - 1 && threads % g.C4 == 0 &&
+                                        (!segmented || (g.sw - 1 + g.pw <= (g.KW - 1) * g.dw &&
+                                                        (g.OW - 1) * g.sw - g.pw + (g.KW - 1) * g.dw >= g.W - 1))));
             if (fuse)
                 *fused = true;
+            const size_t band_row_bytes = (size_t)input_columns_under(g, wseg) * (g.C + 4) * 4;
             size_t lds = deep ? (size_t)deep_lds_bytes(in_rows)
                               : flat ? (size_t)in_rows * kFlatPitch * 4
-                                     : (size_t)in_rows * row_bytes + (size_t)(g.C + 4) * 4; // + the pixel of zeros
+                                     : (size_t)in_rows * band_row_bytes + (size_t)(g.C + 4) * 4; // + the pixel of zeros
             const int bands = flat ? 0 : (g.OH + rb - 1) / rb;
-            const int64_t work_blocks = flat ? (g.M + in_rows - 1) / in_rows : (int64_t)g.N * bands;
+            const int64_t work_blocks =
+                flat ? (g.M + in_rows - 1) / in_rows : (int64_t)g.N * bands * ((g.OW + wseg - 1) / wseg);
             // the filter pre-pass rides along in the same launch (its workgroups want 512 or 1024 threads, so
             // every workgroup gets that many; only `threads` of them take part in the patch sums)
             FilterWork fw = {};
@@ -1469,7 +1580,7 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 // A block of pack work would hold a patch-sum block's worth of LDS for nothing: with bands of rows
                 // (large LDS, most threads idle while the chains run) idle wavefronts of the patch-sum blocks pack,
                 // those on SIMDs that hold no chain, so at most three chain wavefronts per block.
-                if (!flat && rb * g.OW <= 3 * 64)
+                if (!flat && rb * wseg <= 3 * 64)
                     fw.pack_total = total;
                 fw.blocks = fw.sum_blocks + (fw.pack_total > 0 ? 0 : (int)blocks_for(total, block_threads));
                 fw.blocks8 = (fw.blocks + 7) & ~7;
@@ -1481,7 +1592,8 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
             if (e != hipSuccess)
                 return e;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)), dim3(block_threads),
-                               lds, stream, x, g, rb, in_rows, threads, tq, lq_dev, psum, fuse ? xq_fused : nullptr, fw);
+                               lds, stream, x, g, rb, in_rows, threads, wseg, tq, lq_dev, psum,
+                               fuse ? xq_fused : nullptr, fw);
             return hipGetLastError();
         }
     }
