@@ -1528,7 +1528,8 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
         const bool deep = flat && g.C >= 512 && g.M < (int64_t)64 * device_cus();
         if (flat) { // in_rows carries the pixels per workgroup: at least ~2 workgroups per CU where the layer allows
             rb = 0;
-            in_rows = g.M >= 512 * kFlatPixels ? kFlatPixels : (g.M >= 512 * 128 ? 128 : 64);
+            // measured: 128 pixels from 28x28x64 images on (-13 % against 64), 256 only with few channels
+            in_rows = (g.M >= 512 * kFlatPixels && g.C <= 128) ? kFlatPixels : (g.M >= 512 * 64 ? 128 : 64);
         }
         if (deep) {
             rb = -1;
