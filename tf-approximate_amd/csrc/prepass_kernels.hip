@@ -513,10 +513,23 @@ __global__ void __launch_bounds__(1024) patch_sums_smallc_kernel(const float *__
     const int oh0 = (bid - n * bands) * rb;
     const int ih_first = oh0 * g.sh - g.ph;  // input row held in LDS row 0 (may lie outside the image)
     const int row_floats = g.W * g.C;
-    for (int i = t; i < in_rows * row_floats; i += blockDim.x) {
-        const int r = i / row_floats, e = i - r * row_floats;
-        const int ih = ih_first + r;
-        rows[i] = (unsigned)ih < (unsigned)g.H ? fake_quant_value(x[((int64_t)n * g.H + ih) * row_floats + e], qt) : 0.0f;
+    if ((row_floats & 3) == 0 && ((uintptr_t)x & 15) == 0) {   // rows of whole 16-byte pieces (3 x 224, 3 x 32 ...)
+        const int row_quads = row_floats >> 2;
+        for (int i = t; i < in_rows * row_quads; i += blockDim.x) {
+            const int r = i / row_quads, e = i - r * row_quads;
+            const int ih = ih_first + r;
+            float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if ((unsigned)ih < (unsigned)g.H)
+                v = fake_quant_value4(
+                    *reinterpret_cast<const float4 *>(x + ((int64_t)n * g.H + ih) * row_floats + e * 4), qt);
+            *reinterpret_cast<float4 *>(&rows[i * 4]) = v;
+        }
+    } else {
+        for (int i = t; i < in_rows * row_floats; i += blockDim.x) {
+            const int r = i / row_floats, e = i - r * row_floats;
+            const int ih = ih_first + r;
+            rows[i] = (unsigned)ih < (unsigned)g.H ? fake_quant_value(x[((int64_t)n * g.H + ih) * row_floats + e], qt) : 0.0f;
+        }
     }
     __syncthreads();
     if (xq && flat_row_bytes) {
@@ -529,13 +542,18 @@ __global__ void __launch_bounds__(1024) patch_sums_smallc_kernel(const float *__
             const int ih = own_lo + ro;
             const float *src = &rows[(ih - ih_first) * row_floats];
             uint32_t packed = 0;
+            int px = (d * 4) / g.C, c = d * 4 - px * g.C;   // pixel and channel of the dword's first byte
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const int b = d * 4 + k, px = b / g.C, c = b - px * g.C, w = px - pad_left;
+                const int w = px - pad_left;
                 const uint32_t code = (unsigned)w < (unsigned)g.W
                                           ? phys_row(quantize_code(src[w * g.C + c], qt.offset, qt.inv_scale))
                                           : zp;
                 packed |= code << (8 * k);
+                if (++c == g.C) {
+                    c = 0;
+                    ++px;
+                }
             }
             xq[((int64_t)n * g.H + ih) * per_row + d] = packed;
         }
@@ -562,6 +580,18 @@ __global__ void __launch_bounds__(1024) patch_sums_smallc_kernel(const float *__
         return;
     const int iw0 = ow * g.sw - g.pw;
     float s = 0.0f;
+    if (g.dw == 1) {
+        // the taps of a filter row that lie inside the image are one run of floats, in the order of the chain
+        const int lo = (iw0 < 0 ? 0 : iw0) * g.C, hi = (iw0 + g.KW < g.W ? iw0 + g.KW : g.W) * g.C;
+        for (int kh = 0; kh < g.KH; ++kh) {
+            const float *src = &rows[(ohl * g.sh + kh * g.dh) * row_floats];   // rows outside the image hold zeros
+#pragma unroll 4
+            for (int j = lo; j < hi; ++j)
+                s = __fadd_rn(s, src[j]);
+        }
+        psum[((int64_t)n * g.OH + oh) * g.OW + ow] = s;
+        return;
+    }
     for (int kh = 0; kh < g.KH; ++kh) {
         const int r = ohl * g.sh + kh * g.dh;        // LDS row of this tap; rows outside the image hold zeros
         for (int kw = 0; kw < g.KW; ++kw) {
