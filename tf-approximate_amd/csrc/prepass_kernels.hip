@@ -1013,25 +1013,47 @@ __device__ __forceinline__ void patch_sums_deep_body(const float *__restrict__ x
         psum[m0 + t] = s;
 }
 
+// The filter work of the first fw.blocks8 workgroups of a patch-sum launch.
+__device__ __forceinline__ void filter_work_block(const FilterWork &fw, const LayerQuant *__restrict__ lq_dev)
+{
+    if ((int)blockIdx.x >= fw.blocks)
+        return;
+    const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
+    if ((int)blockIdx.x < fw.sum_blocks) { // the launcher gives these workgroups 512 or 1024 threads
+        if (blockDim.x == 512)
+            filter_sums_block<512>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
+        else
+            filter_sums_block<1024>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
+        return;
+    }
+    const int64_t i = (int64_t)((int)blockIdx.x - fw.sum_blocks) * blockDim.x + threadIdx.x;
+    filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+}
+
+// Bands cut into column segments: a kernel of its own, so that the common variants below stay as small as they were.
+__global__ void __launch_bounds__(1024) patch_sums_segments_kernel(const float *__restrict__ x, const ConvGeom g,
+                                                                    int rb, int in_rows, int nthreads, int wseg,
+                                                                    const TensorQuant tq,
+                                                                    const LayerQuant *__restrict__ lq_dev,
+                                                                    float *__restrict__ psum, uint32_t *__restrict__ xq,
+                                                                    const FilterWork fw)
+{
+    if ((int)blockIdx.x < fw.blocks8) {
+        filter_work_block(fw, lq_dev);
+        return;
+    }
+    patch_sums_rows_body<true>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
+                               (int)gridDim.x - fw.blocks8, nthreads, fw);
+}
+
 __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, const ConvGeom g, int rb,
-                                                                int in_rows, int nthreads, int wseg, const TensorQuant tq,
+                                                                int in_rows, int nthreads, const TensorQuant tq,
                                                                 const LayerQuant *__restrict__ lq_dev,
                                                                 float *__restrict__ psum, uint32_t *__restrict__ xq,
                                                                 const FilterWork fw)
 {
     if ((int)blockIdx.x < fw.blocks8) {
-        if ((int)blockIdx.x >= fw.blocks)
-            return;
-        const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
-        if ((int)blockIdx.x < fw.sum_blocks) { // the launcher gives these workgroups 512 or 1024 threads
-            if (blockDim.x == 512)
-                filter_sums_block<512>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
-            else
-                filter_sums_block<1024>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
-            return;
-        }
-        const int64_t i = (int64_t)((int)blockIdx.x - fw.sum_blocks) * blockDim.x + threadIdx.x;
-        filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+        filter_work_block(fw, lq_dev);
         return;
     }
     if (rb < 0) { // 1x1, stride 1, many channels, few pixels
@@ -1045,12 +1067,8 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
         patch_sums_flat_body(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8, in_rows);
         return;
     }
-    if (wseg >= g.OW)
-        patch_sums_rows_body<false>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
-                                    (int)gridDim.x - fw.blocks8, nthreads, fw);
-    else
-        patch_sums_rows_body<true>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
-                                   (int)gridDim.x - fw.blocks8, nthreads, fw);
+    patch_sums_rows_body<false>(x, g, rb, in_rows, g.OW, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
+                                (int)gridDim.x - fw.blocks8, nthreads, fw);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -1619,12 +1637,21 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                     lds = kFsLdsBytes;
                 *filter_done = true;
             }
+            if (segmented) {
+                const hipError_t e =
+                    set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_segments_kernel), 160 * 1024);
+                if (e != hipSuccess)
+                    return e;
+                hipLaunchKernelGGL(patch_sums_segments_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)),
+                                   dim3(block_threads), lds, stream, x, g, rb, in_rows, threads, wseg, tq, lq_dev, psum,
+                                   fuse ? xq_fused : nullptr, fw);
+                return hipGetLastError();
+            }
             const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_rows_kernel), 160 * 1024);
             if (e != hipSuccess)
                 return e;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)), dim3(block_threads),
-                               lds, stream, x, g, rb, in_rows, threads, wseg, tq, lq_dev, psum,
-                               fuse ? xq_fused : nullptr, fw);
+                               lds, stream, x, g, rb, in_rows, threads, tq, lq_dev, psum, fuse ? xq_fused : nullptr, fw);
             return hipGetLastError();
         }
     }
