@@ -229,8 +229,8 @@ __global__ void __launch_bounds__(kPsTile) patch_sums_tiled_kernel(const float *
 }
 
 // The filter pre-pass of a layer is independent of its input pre-pass: as two launches they would run one after
-// the other, so the launch below carries both.  The first filter_blocks8 workgroups (a multiple of 8, which keeps
-// workgroup index mod 8 = XCD for the others) do the filter work of filter_prep_kernel, the rest the patch sums.
+// the other, so the launch below carries both: the filter work of filter_prep_kernel in workgroups of its own
+// (ordered as described at the members below), the patch sums in the others.
 struct FilterWork {
     const float *filter;
     const uint8_t *filter_codes;
@@ -239,8 +239,12 @@ struct FilterWork {
     uint16_t *wq;
     int sum_blocks;
     float *fsum;
-    int blocks;    // sum_blocks + pack blocks; 0: no filter work in this launch
-    int blocks8;   // blocks rounded up to a multiple of 8
+    // Order of the workgroups of a launch: the filter sums (long chains: first), rounded up to a multiple of 8 so
+    // that workgroup index mod 8 stays the XCD for the others; the patch sums; the workgroups that pack filter codes
+    // (many and short: they fill the tail).
+    int sum8;         // sum_blocks rounded up to a multiple of 8
+    int work_blocks;  // patch-sum workgroups
+    int pack_blocks;  // 0: no pack workgroups
     // pack_total > 0: no pack blocks; the threads of the patch-sum blocks that run no chain pack the codes,
     // each block its share of the pack_total elements
     int64_t pack_total;
@@ -1013,21 +1017,28 @@ __device__ __forceinline__ void patch_sums_deep_body(const float *__restrict__ x
         psum[m0 + t] = s;
 }
 
-// The filter work of the first fw.blocks8 workgroups of a patch-sum launch.
-__device__ __forceinline__ void filter_work_block(const FilterWork &fw, const LayerQuant *__restrict__ lq_dev)
+// The filter work of a patch-sum launch: true if this workgroup is one of those that do it (and has done it), else
+// *bid is its index among the patch-sum workgroups.
+__device__ __forceinline__ bool filter_work_block(const FilterWork &fw, const LayerQuant *__restrict__ lq_dev, int *bid)
 {
-    if ((int)blockIdx.x >= fw.blocks)
-        return;
-    const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
-    if ((int)blockIdx.x < fw.sum_blocks) { // the launcher gives these workgroups 512 or 1024 threads
-        if (blockDim.x == 512)
-            filter_sums_block<512>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
-        else
-            filter_sums_block<1024>((int)blockIdx.x, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
-        return;
+    const int b = (int)blockIdx.x;
+    if (b < fw.sum8) {
+        if (b < fw.sum_blocks) { // the launcher gives these workgroups 512 or 1024 threads
+            const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
+            if (blockDim.x == 512)
+                filter_sums_block<512>(b, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
+            else
+                filter_sums_block<1024>(b, fw.filter, fw.taps * fw.C, fw.Co, q, fw.fsum);
+        }
+        return true;
     }
-    const int64_t i = (int64_t)((int)blockIdx.x - fw.sum_blocks) * blockDim.x + threadIdx.x;
+    *bid = b - fw.sum8;
+    if (*bid < fw.work_blocks)
+        return false;
+    const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
+    const int64_t i = (int64_t)(*bid - fw.work_blocks) * blockDim.x + threadIdx.x;
     filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+    return true;
 }
 
 // Bands cut into column segments: a kernel of its own, so that the common variants below stay as small as they were.
@@ -1038,12 +1049,10 @@ __global__ void __launch_bounds__(1024) patch_sums_segments_kernel(const float *
                                                                     float *__restrict__ psum, uint32_t *__restrict__ xq,
                                                                     const FilterWork fw)
 {
-    if ((int)blockIdx.x < fw.blocks8) {
-        filter_work_block(fw, lq_dev);
+    int bid;
+    if (filter_work_block(fw, lq_dev, &bid))
         return;
-    }
-    patch_sums_rows_body<true>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
-                               (int)gridDim.x - fw.blocks8, nthreads, fw);
+    patch_sums_rows_body<true>(x, g, rb, in_rows, wseg, tq, lq_dev, psum, xq, bid, fw.work_blocks, nthreads, fw);
 }
 
 __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__restrict__ x, const ConvGeom g, int rb,
@@ -1052,23 +1061,21 @@ __global__ void __launch_bounds__(1024) patch_sums_rows_kernel(const float *__re
                                                                 float *__restrict__ psum, uint32_t *__restrict__ xq,
                                                                 const FilterWork fw)
 {
-    if ((int)blockIdx.x < fw.blocks8) {
-        filter_work_block(fw, lq_dev);
+    int bid;
+    if (filter_work_block(fw, lq_dev, &bid))
         return;
-    }
     if (rb < 0) { // 1x1, stride 1, many channels, few pixels
         if (in_rows == 8)
-            patch_sums_deep_body<8>(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8);
+            patch_sums_deep_body<8>(x, g, tq, lq_dev, psum, xq, bid);
         else
-            patch_sums_deep_body<16>(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8);
+            patch_sums_deep_body<16>(x, g, tq, lq_dev, psum, xq, bid);
         return;
     }
     if (rb == 0) { // 1x1, stride 1: flat pixel list
-        patch_sums_flat_body(x, g, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8, in_rows);
+        patch_sums_flat_body(x, g, tq, lq_dev, psum, xq, bid, in_rows);
         return;
     }
-    patch_sums_rows_body<false>(x, g, rb, in_rows, g.OW, tq, lq_dev, psum, xq, (int)blockIdx.x - fw.blocks8,
-                                (int)gridDim.x - fw.blocks8, nthreads, fw);
+    patch_sums_rows_body<false>(x, g, rb, in_rows, g.OW, tq, lq_dev, psum, xq, bid, fw.work_blocks, nthreads, fw);
 }
 
 __global__ void __launch_bounds__(256) quantize_flat_kernel(const float *__restrict__ v, int64_t n, float offset,
@@ -1631,26 +1638,27 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 // those on SIMDs that hold no chain, so at most three chain wavefronts per block.
                 if (!flat && rb * wseg <= 3 * 64)
                     fw.pack_total = total;
-                fw.blocks = fw.sum_blocks + (fw.pack_total > 0 ? 0 : (int)blocks_for(total, block_threads));
-                fw.blocks8 = (fw.blocks + 7) & ~7;
+                fw.sum8 = (fw.sum_blocks + 7) & ~7;
+                fw.pack_blocks = fw.pack_total > 0 ? 0 : (int)blocks_for(total, block_threads);
                 if (fw.sum_blocks && lds < (size_t)kFsLdsBytes)
                     lds = kFsLdsBytes;
                 *filter_done = true;
             }
+            fw.work_blocks = (int)work_blocks;
+            const unsigned grid = (unsigned)(fw.sum8 + work_blocks + fw.pack_blocks);
             if (segmented) {
                 const hipError_t e =
                     set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_segments_kernel), 160 * 1024);
                 if (e != hipSuccess)
                     return e;
-                hipLaunchKernelGGL(patch_sums_segments_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)),
-                                   dim3(block_threads), lds, stream, x, g, rb, in_rows, threads, wseg, tq, lq_dev, psum,
+                hipLaunchKernelGGL(patch_sums_segments_kernel, dim3(grid), dim3(block_threads), lds, stream, x, g, rb, in_rows, threads, wseg, tq, lq_dev, psum,
                                    fuse ? xq_fused : nullptr, fw);
                 return hipGetLastError();
             }
             const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_rows_kernel), 160 * 1024);
             if (e != hipSuccess)
                 return e;
-            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3((unsigned)(fw.blocks8 + work_blocks)), dim3(block_threads),
+            hipLaunchKernelGGL(patch_sums_rows_kernel, dim3(grid), dim3(block_threads),
                                lds, stream, x, g, rb, in_rows, threads, tq, lq_dev, psum, fuse ? xq_fused : nullptr, fw);
             return hipGetLastError();
         }
