@@ -76,19 +76,19 @@ LAYERS = [
 # device copy of known size inside the same run.  Keyed by (workload, kernel); not measured in the run that prints
 # them: the bench line says which profile they come from.
 PROFILED_TRAFFIC = {
-    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 80844.6 * 1024 + 1.000 * 61112.4 * 1024,
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 80848.9 * 1024 + 1.000 * 62076.4 * 1024,
                                                            "profiles/lutgemm_px_conv3x3_b64_56x56x64.md"),
-    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8312.5 * 1024 + 1.000 * 61291.7 * 1024,
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8312.5 * 1024 + 1.000 * 61757.9 * 1024,
                                                                "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
-    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48276.2 * 1024 + 1.000 * 785480.6 * 1024,
+    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48275.5 * 1024 + 1.000 * 784460.2 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b64_112x112x32_to_192.md"),
-    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37214.5 * 1024 + 1.000 * 262929.9 * 1024,
+    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37242.1 * 1024 + 1.000 * 262539.4 * 1024,
                                                     "profiles/lutgemm_px_conv1x1_b64_56x56x64_to_256.md"),
-    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 466401.3 * 1024 + 1.000 * 498705.7 * 1024,
+    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 466401.4 * 1024 + 1.000 * 503985.5 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
-    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 92846.2 * 1024 + 1.000 * 271937.5 * 1024,
+    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 92846.3 * 1024 + 1.000 * 272367.6 * 1024,
                                                       "profiles/lutgemm_px_conv7x7s2_b64_224x224x3_to_64.md"),
-    ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51701.6 * 1024 + 1.000 * 106125.5 * 1024,
+    ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51701.5 * 1024 + 1.000 * 106261.2 * 1024,
                                                          "profiles/lutgemm_expand_conv3x3_b64_28x28x512_to_512.md"),
     ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6128.5 * 1024 + 1.025 * 8192.0 * 1024,
                                                     "profiles/lutgemm_px_conv3x3_b128_32x32x16_to_16.md"),
