@@ -90,6 +90,33 @@ def test_extreme_shapes_vs_oracle(pkg, oracle, case):
     assert refimpl.linf_rel(y, y_ref) <= 1e-5, case
 
 
+WIDE_ROWS = [
+    # rows of many channels: the patch sums hold only a column segment of every band in LDS (whole rows would leave
+    # one workgroup per CU, or not fit at all); inputs off the quantization grid, so the order of the sums counts
+    ((30, 20, 41, 256), (3, 3, 256, 8), (1, 1), (1, 1), "SAME"),     # odd width, padding on both sides
+    ((48, 21, 40, 256), (3, 3, 256, 8), (2, 2), (1, 1), "SAME"),     # stride 2: padding after only
+    ((40, 17, 50, 192), (3, 5, 192, 8), (1, 3), (1, 2), "SAME"),     # stride 3 and dilation 2 along the row
+    ((6, 19, 37, 320), (5, 3, 320, 8), (2, 1), (2, 1), "VALID"),     # no padding, dilated and strided rows
+    ((3, 12, 30, 512), (3, 3, 512, 16), (1, 1), (1, 1), "SAME"),     # three rows do not fit LDS: long chains
+    ((2, 9, 26, 1024), (3, 3, 1024, 8), (1, 1), (1, 1), "SAME"),     # ... nor does one row twice
+]
+
+
+@pytest.mark.parametrize("case", WIDE_ROWS, ids=[str(i) for i in range(len(WIDE_ROWS))])
+def test_wide_rows_of_many_channels_vs_oracle(pkg, oracle, case):
+    xs, fs, strides, dil, padding = case
+    mm = (-1.0, 1.0, -0.5, 0.5)
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, mm, seed=len(str(case)))
+    x = (x + np.float32(0.0013)).astype(np.float32)
+    table = pkg.synth.table_random(3)
+    y, acc = gpu_util.run_op(pkg, table, x, f, mm, strides, padding, dil)
+    rc, y_ref, acc_ref = oracle.conv2d_fast(table, x, f, *mm, strides=strides, padding=padding, dilations=dil,
+                                            threads=8)
+    assert rc == 0
+    assert np.array_equal(acc, acc_ref), case
+    assert np.array_equal(y, y_ref), case     # the same sums in the same order: no tolerance needed
+
+
 @pytest.mark.parametrize("columns", [32, 64])
 def test_wider_column_tiles_vs_oracle(pkg, oracle, columns):
     """The tile planner has so far always chosen 16-column tiles; the 32- and 64-column variants of the kernel
