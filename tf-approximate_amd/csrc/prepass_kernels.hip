@@ -412,6 +412,7 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
         return;
     const int iw0 = ow * g.sw - g.pw;
     float s = 0.0f;
+    __builtin_amdgcn_s_setprio(3);   // the chain is the critical path: its wavefront issues ahead of the others on its SIMD
     if ((g.C4 & 7) == 0) {
         // The chain of K dependent adds is what takes the time here, so nothing else may wait on it: the taps and
         // their channels form one flat list of batches of 32 floats, the LDS reads of a batch are issued a batch
@@ -721,6 +722,7 @@ __device__ __forceinline__ void filter_sums_block(const int block, const float *
     issue(v[0], kFsAhead);
     __syncthreads();
     float s = 0.0f;
+    __builtin_amdgcn_s_setprio(3);   // the chain is the critical path: its wavefront issues ahead of the others on its SIMD
     // one pass: `next` holds pass p + 1 (stored now, then refilled with the loads of pass p + 1 + kFsAhead);
     // pass p lies in its half of the stage
     auto pass_step = [&](const int p, float(&next)[kPer]) {
@@ -843,6 +845,7 @@ __device__ __forceinline__ void patch_sums_flat_body(const float *__restrict__ x
     };
     load_chunk(0);
     float s = 0.0f;
+    __builtin_amdgcn_s_setprio(3);   // the chain is the critical path: its wavefront issues ahead of the others on its SIMD
     for (int ch = 0; ch < chunks; ++ch) {
         const int c0 = ch * kFlatChunk;
         if (copier) {
@@ -963,6 +966,7 @@ __device__ __forceinline__ void patch_sums_deep_body(const float *__restrict__ x
         issue(v[0], kDeepAhead);
     __syncthreads();
     float s = 0.0f;
+    __builtin_amdgcn_s_setprio(3);   // the chain is the critical path: its wavefront issues ahead of the others on its SIMD
     constexpr int kBatch = 8, kBatches = QUADS / kBatch; // 16-byte reads per batch; batches per pass
     auto pass_step = [&](const int p, float4(&next)[kDeepPer]) {
         store(next, p + 1);
