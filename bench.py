@@ -9,11 +9,12 @@ fused epilogue) on seeded synthetic tensors that are already resident in HBM.  P
   value        approximate GMAC/s of the whole op (1 MAC = 1 truth-table lookup) on the headline layer, wall clock
                over K steps
   roofline     the LUT-GEMM kernel alone: algorithmic lookups per launch / its mean launch duration (HIP events on
-               the launch stream, recorded inside the library), as a fraction of the two ceilings that can bind it,
-               both measured in this run: the LDS read port (streaming ds_read_b128; a lookup moves its 2-byte
-               entry through it) and the issue rate of the kernel's accumulate instructions.  `frac` is the larger
-               of the two, `peak` the ceiling it belongs to; `frac_nominal_gather` is the same rate against the
-               nominal one-entry-per-bank-slot gather ceiling 256 CU x 32 lookups/clk x 2.4 GHz = 19.66 T/s.
+               the launch stream, recorded inside the library), as a fraction of the two ceilings that can bind it:
+               the LDS read port (a lookup moves its 2-byte entry through it) and the issue rate of the kernel's
+               accumulate instructions, each the larger of its nominal value (CUs x 256 B x clock, CUs x 64 lanes x
+               clock) and what a probe kernel measures in this run.  `frac` is the larger of the two fractions,
+               `peak` the ceiling it belongs to; `frac_nominal_gather` is the same rate against the nominal
+               one-entry-per-bank-slot gather ceiling 256 CU x 32 lookups/clk x 2.4 GHz = 19.66 T/s.
   layers       the same measurement for the layer shapes of the other benchmark configurations (fewer steps each),
                every one with an oracle check of sampled output pixels; depthwise layers against HBM bandwidth
   networks     images/s of the two synthetic ResNet-shaped networks, every convolution through the op
@@ -69,7 +70,10 @@ LAYERS = [
     ("cfg4_resnet50", "stage4_1x1_512_2048", (64, 7, 7, 512), (1, 1, 512, 2048), (1, 1), False, "uniform", "uniform_error"),
     ("cfg5_stress", "A_1x1_256_1024", (32, 56, 56, 256), (1, 1, 256, 1024), (1, 1), False, "halfnormal", "random"),
     ("cfg5_stress", "B_3x3_512_512", (64, 28, 28, 512), (3, 3, 512, 512), (1, 1), False, "halfnormal", "random"),
+    ("cfg5_stress", "A_1x1_256_1024", (32, 56, 56, 256), (1, 1, 256, 1024), (1, 1), False, "halfnormal", "exact"),
+    ("cfg5_stress", "B_3x3_512_512", (64, 28, 28, 512), (3, 3, 512, 512), (1, 1), False, "halfnormal", "exact"),
 ]
+CPU_SAMPLE_S = 0.5      # single-thread reference sample per `layers` record
 
 # Bytes per launch that the main kernel moves between its L2s and the memory side (Infinity Cache or HBM), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each scaled by what the same counter reads for the
@@ -117,7 +121,9 @@ def measured_copy_bandwidth(mib=512, reps=30):
 
 
 class Ceilings:
-    """The ceilings of the dense kernel, measured once per run."""
+    """The ceilings of the dense kernel: measured once per run by probe kernels of the library, and nominal from the
+    device's CU count and clock.  A fraction is taken against the LARGER of the two, so a probe that falls short of
+    what the hardware is specified for does not flatter the kernel."""
 
     def __init__(self, ops):
         self.copy_bytes = measured_copy_bandwidth()
@@ -125,22 +131,34 @@ class Ceilings:
         self.port_bytes = max(ops.lds_read_peak(), 1.0)         # streaming ds_read_b128 bytes/s
         self.valu_lane_ops = max(ops.valu_issue_peak(), 1.0)    # accumulate-instruction lane operations/s
         self.ops_per_lookup = ops.dense_accumulate_ops_per_lookup()
+        info = ops.device_info()
+        self.cus, self.clock_hz = info["compute_units"], info["clock_khz"] * 1e3
+        self.valu_nominal = self.cus * 64.0 * self.clock_hz     # 4 SIMDs x 16 lanes per clock and CU
+        self.port_nominal = self.cus * 256.0 * self.clock_hz    # 64 banks x 4 bytes per clock and CU
 
     def fractions(self, lookups_per_s):
-        f_port = 2.0 * lookups_per_s / self.port_bytes
-        f_valu = lookups_per_s * self.ops_per_lookup / self.valu_lane_ops
+        valu_ceiling = max(self.valu_nominal, self.valu_lane_ops)
+        port_ceiling = max(self.port_nominal, self.port_bytes)
+        f_port = 2.0 * lookups_per_s / port_ceiling
+        f_valu = lookups_per_s * self.ops_per_lookup / valu_ceiling
         bound = "lds" if f_port >= f_valu else "valu"
-        peak = self.port_bytes / 2.0 if bound == "lds" else self.valu_lane_ops / self.ops_per_lookup
+        peak = port_ceiling / 2.0 if bound == "lds" else valu_ceiling / self.ops_per_lookup
         return {"bound": bound, "frac": round(max(f_port, f_valu), 4), "frac_lds_port": round(f_port, 4),
                 "frac_valu": round(f_valu, 4),
+                "frac_lds_port_measured": round(2.0 * lookups_per_s / self.port_bytes, 4),
+                "frac_valu_measured": round(lookups_per_s * self.ops_per_lookup / self.valu_lane_ops, 4),
                 "frac_nominal_gather": round(lookups_per_s / NOMINAL_LDS_LOOKUPS_PER_S, 4)}, peak
 
     def report(self):
-        return {"lds_read_port_gbytes_per_s": round(self.port_bytes / 1e9, 1),
+        return {"compute_units": self.cus, "clock_ghz": round(self.clock_hz / 1e9, 3),
+                "valu_nominal_glane_ops_per_s": round(self.valu_nominal / 1e9, 1),
+                "lds_port_nominal_gbytes_per_s": round(self.port_nominal / 1e9, 1),
+                "lds_read_port_gbytes_per_s": round(self.port_bytes / 1e9, 1),
                 "lds_read_port_glookups_per_s": round(self.port_bytes / 2e9, 1),
                 "valu_accumulate_glane_ops_per_s": round(self.valu_lane_ops / 1e9, 1),
                 "valu_ops_per_lookup": self.ops_per_lookup,
                 "valu_glookups_per_s": round(self.valu_lane_ops / self.ops_per_lookup / 1e9, 1),
+                "valu_nominal_glookups_per_s": round(self.valu_nominal / self.ops_per_lookup / 1e9, 1),
                 "nominal_gather_glookups_per_s": round(NOMINAL_LDS_LOOKUPS_PER_S / 1e9, 1),
                 "measured_ds_read_u16_glookups_per_s": round(self.gather / 1e9, 1),
                 "hbm_device_copy_gbytes_per_s": round(self.copy_bytes / 1e9, 1)}
@@ -271,6 +289,35 @@ def dense_kernel_name(kernels_ms):
     return "lutgemm_px" if "lutgemm_px" in kernels_ms else "lutgemm_expand"
 
 
+def cpu_reference_sample(oracle, table, xd, fd, strides, depthwise, seconds=CPU_SAMPLE_S):
+    """The oracle's reference-faithful single-thread path on the first output pixels of the first image, sized for
+    about `seconds` of work, and its OpenMP variant on the first image; GMAC/s each.  The reference has no depthwise
+    op: there the oracle's definition (the dense path per channel) runs on the first rows of the first image."""
+    x1 = xd[:1].cpu().numpy()
+    f = fd.cpu().numpy()
+    cores = max(1, min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "64"))))
+    if depthwise:
+        rows = min(x1.shape[1], 8 * strides[0])
+        t0 = time.perf_counter()
+        rc, y, _ = oracle.depthwise_conv2d(table, x1[:, :rows], f, *MM, strides=strides, padding="SAME")
+        secs = time.perf_counter() - t0
+        macs = y.size * f.shape[0] * f.shape[1]
+        return {"cpu_ref_1t_gmacs": round(macs / secs / 1e9, 4), "cpu_omp_gmacs": None, "host_cores": cores,
+                "cpu_sample": "first %d input rows of image 0, the dense reference path per channel" % rows}
+    kh, kw, c, co = f.shape
+    per_pixel = co * kh * kw * c
+    _, d = oracle.geometry(x1.shape, f.shape, strides, "SAME")
+    pixels_image = int(d.out_rows) * int(d.out_cols)
+    patches = int(max(4, min(pixels_image, seconds * 0.4e9 / per_pixel)))
+    secs, _ = oracle.time_reference_chunk(table, x1, f, *MM, patches, strides=strides, padding="SAME")
+    t0 = time.perf_counter()
+    rc, _, _ = oracle.conv2d_fast(table, x1, f, *MM, strides=strides, padding="SAME", threads=cores)
+    t_omp = time.perf_counter() - t0
+    return {"cpu_ref_1t_gmacs": round(patches * per_pixel / secs / 1e9, 4),
+            "cpu_omp_gmacs": round(pixels_image * per_pixel / t_omp / 1e9, 3) if rc == 0 else None, "host_cores": cores,
+            "cpu_sample": "first %d output pixels of image 0 (1 thread, extrapolates to the layer); image 0 (OpenMP)" % patches}
+
+
 def measure_layer(pkg, ops, oracle, ceil, spec, steps=None, preroll_s=0.08):
     config, name, xs, fs, strides, depthwise, codes, tkind = spec
     table = make_table(pkg.synth, tkind)
@@ -301,6 +348,7 @@ def measure_layer(pkg, ops, oracle, ceil, spec, steps=None, preroll_s=0.08):
         exact, linf = sampled_oracle_check(oracle, table, op, xd, fd, strides, depthwise, y)
         rec["acc_bit_exact"] = exact
         rec["linf_rel"] = linf
+        rec.update(cpu_reference_sample(oracle, table, xd, fd, strides, depthwise))
     rec["kernels_ms"] = {k: round(v, 4) for k, v in sorted(kms.items())}
     del xd, fd, y
     return rec
@@ -473,16 +521,20 @@ def main():
             "frac": fr["frac"],
             "frac_lds_port": fr["frac_lds_port"],
             "frac_valu": fr["frac_valu"],
+            "frac_lds_port_measured": fr["frac_lds_port_measured"],
+            "frac_valu_measured": fr["frac_valu_measured"],
             "frac_nominal_gather": fr["frac_nominal_gather"],
             "traffic": traffic,
             "traffic_source": traffic_source,
             "kernel_ms": round(main_ms, 4),
             "lookups_per_launch": lookups,
             "ceilings": ceil.report(),
-            "note": "frac = the larger of frac_lds_port (2 bytes per lookup against the measured streaming "
-                    "ds_read_b128 rate) and frac_valu (accumulate instructions per lookup against their measured "
-                    "issue rate); frac_nominal_gather is against 256 CU x 32 lookups/clk x 2.4 GHz, a ceiling for "
-                    "one-entry gathers that a kernel reading 8 entries per access can pass",
+            "note": "frac = the larger of frac_lds_port (2 bytes per lookup against the LDS read port) and frac_valu "
+                    "(accumulate instructions per lookup against the vector ALUs' issue rate), each against the larger "
+                    "of its nominal ceiling (CUs x 256 B x clock; CUs x 64 lanes x clock) and the rate a probe kernel "
+                    "measured in this run; the *_measured figures are against the probes alone; frac_nominal_gather "
+                    "is against 256 CU x 32 lookups/clk x 2.4 GHz, a ceiling for one-entry gathers that a kernel "
+                    "reading 8 entries per access can pass",
             "hbm_algorithmic_bytes": hbm_bytes,
             "hbm_gbps_whole_op": round(hbm_bytes / (ms_per_step * 1e-3) / 1e9, 1),
             "hbm_frac_whole_op": round(hbm_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
@@ -552,7 +604,9 @@ def main():
     if not args.no_networks:
         t_n = time.perf_counter()
         result["networks"] = [measure_network(pkg, "cifar_resnet_b128", 40, 10),
-                              measure_network(pkg, "resnet50_b64", 12, 3)]
+                              measure_network(pkg, "resnet50_b64", 12, 3),
+                              measure_network(pkg, "cifar_resnet_b128", 40, 10, fused_layers=True),
+                              measure_network(pkg, "resnet50_b64", 12, 3, fused_layers=True)]
         result["networks_seconds"] = round(time.perf_counter() - t_n, 1)
     print(json.dumps(result))
 

@@ -148,12 +148,13 @@ int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[8]);
  * value and is read once, when the library is loaded.  Like axc_set_preexpand it is process-wide; a workspace query and
  * the launch it is for must see the same value. */
 int axc_set_tile_columns(int columns);
-/* Layers with many output pixels per filter element (16-column tiles, no K split, an even number of channel quads,
- * at most 192 MiB of rows) run out of pre-expanded rows: the table rows of every filter element are laid out in the
+/* Layers with many output pixels per filter element (16-column tiles, an even number of channel quads, whole pairs
+ * of fills per K split where K is split, at most 192 MiB of rows) run out of pre-expanded rows: the table rows of every filter element are laid out in the
  * workspace once per call instead of inside every tile.  mode 0 = the planner decides (the default), 1 = every
  * layer that can run that way does, -1 = none does; process-wide, for tests and timing, initial value from the
  * environment variable AXC_PREEXPAND (read once, when the library is loaded).  Results do not depend on it.  The
- * workspace query counts the rows; a launch whose workspace lacks room for them runs without them.  No counterpart
+ * workspace query counts the rows; a launch whose workspace lacks room for them runs without them, with the tile
+ * plan of the kernel that expands inside its tiles when the workspace holds what that plan needs.  No counterpart
  * in the reference. */
 int axc_set_preexpand(int mode);
 int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
@@ -185,8 +186,7 @@ int axc_depthwise_conv2d_minmax_bias_act(const axc_table *table, const axc_conv2
                                          float *output, void *workspace, size_t workspace_bytes, void *stream);
 
 /* axc_conv2d_minmax for callers that cannot allocate or own a workspace (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose launcher allocates its
- * temporaries per call (approx_nn_conv_ops.cpp:590-613).  The workspace is a fixed array of
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is a fixed array of
  * axc_conv2d_static_workspace_limit() bytes (32 MiB) inside the library's device image, one copy per GPU, held
  * until the process ends; the call itself allocates and frees nothing.  Layers whose
  * axc_conv2d_workspace_bytes exceeds the limit are refused with AXC_INVALID_ARGUMENT.  All calls on one GPU

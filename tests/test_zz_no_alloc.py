@@ -57,6 +57,36 @@ def test_static_workspace_entry_point_matches_on_two_calls(pkg, oracle):
     assert rc == 0 and refimpl.linf_rel(got, y_ref) <= 1e-5
 
 
+def test_static_workspace_calls_allocate_nothing(pkg):
+    """Free device memory as the runtime reports it is the same before and after calls of the static entry point
+    (after one warm-up call, which may load the kernels' code), with per-kernel profiling off and on."""
+    from tf_approximate_amd import _lib, ops
+    lib = _lib.load()
+    table = ops.TruthTable(pkg.synth.table_random(6))
+    xs, fs = (4, 14, 14, 256), (3, 3, 256, 64)     # K split: the widest use of the workspace
+    x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=21)
+    dev = torch.device("cuda:0")
+    xd, fd = torch.from_numpy(x).to(dev), torch.from_numpy(f).to(dev)
+    desc = ops.make_desc(xs, fs, [1, 1, 1, 1], "SAME")
+    out = torch.empty((4, 14, 14, 64), dtype=torch.float32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def call():
+        rc = lib.axc_conv2d_minmax_static(table.handle, ctypes.byref(desc), xd.data_ptr(), fd.data_ptr(), *MM,
+                                          out.data_ptr(), stream)
+        assert rc == 0, lib.axc_last_error()
+
+    call()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(dev)
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(dev)
+    assert free_after == free_before, "the static entry point changed free device memory by %d bytes" % (
+        free_before - free_after)
+
+
 def test_static_workspace_refuses_layers_beyond_its_limit(pkg):
     from tf_approximate_amd import _lib, ops
     lib = _lib.load()

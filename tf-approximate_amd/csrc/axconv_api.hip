@@ -44,6 +44,33 @@ int device_cus()
     cached[slot].store(cus, std::memory_order_relaxed);
     return cus;
 }
+
+// LDS a workgroup may take and the shader clock of the current device, as the runtime reports them (cached); the
+// gfx950 figures where it reports nothing.
+static int device_attribute_cached(std::atomic<int> (&cached)[64], hipDeviceAttribute_t attr, int fallback)
+{
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return fallback;
+    const int slot = dev & 63;
+    v = cached[slot].load(std::memory_order_relaxed);
+    if (v > 0)
+        return v;
+    if (hipDeviceGetAttribute(&v, attr, dev) != hipSuccess || v <= 0)
+        return fallback;
+    cached[slot].store(v, std::memory_order_relaxed);
+    return v;
+}
+int device_lds_bytes()
+{
+    static std::atomic<int> cached[64];
+    return device_attribute_cached(cached, hipDeviceAttributeMaxSharedMemoryPerBlock, 160 * 1024);
+}
+double device_clock_hz()
+{
+    static std::atomic<int> cached[64];
+    return 1e3 * (double)device_attribute_cached(cached, hipDeviceAttributeClockRate, 2400000);
+}
 } // namespace axc
 
 namespace {
@@ -353,7 +380,7 @@ constexpr size_t kPxMaxBytes = (size_t)192 << 20;   // most memory a layer's pre
 
 // Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
 // Derive cost per fill is constant; lookup cost per fill grows with the wavefront-rows a SIMD carries.
-DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
+DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode, double clock_hz)
 {
     DensePlan best{};
     double best_cost = 1e300;
@@ -422,7 +449,7 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
                     double px_cost = (double)rounds * ((double)(fps / 2) * (1900.0 + per_simd * 530.0) + 12000.0);
                     if (ks > 1)
                         px_cost = px_cost * 1.08 + split_cost;
-                    px_cost += (6.5e-6 + px_bytes / 5e12) * 2.4e9;
+                    px_cost += (6.5e-6 + px_bytes / 5e12) * clock_hz;
                     if (px_mode > 0 || px_cost < cost) {
                         cost = px_cost;
                         px = 1;
@@ -449,7 +476,8 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode)
 
 // The plan depends on (taps, channel quads, columns, pixels, CUs, forced width) only: looked up instead of
 // recomputed on every workspace query and launch.
-DensePlan make_plan(const ConvGeom &g, int cus)
+constexpr int kPxModeGlobal = 99;   // "whatever axc_set_preexpand says"
+DensePlan make_plan(const ConvGeom &g, int cus, int px_mode = kPxModeGlobal)
 {
     struct Key {
         int taps, c4, co, cus, forced, px_mode;
@@ -463,14 +491,14 @@ DensePlan make_plan(const ConvGeom &g, int cus)
     static std::mutex mu;
     static std::map<Key, DensePlan> cache;
     const Key key{g.KH * g.KW, g.C4, g.Co, cus, g_forced_nt.load(std::memory_order_relaxed),
-                  g_px_mode.load(std::memory_order_relaxed), g.M};
+                  px_mode == kPxModeGlobal ? g_px_mode.load(std::memory_order_relaxed) : px_mode, g.M};
     {
         std::lock_guard<std::mutex> lock(mu);
         auto it = cache.find(key);
         if (it != cache.end())
             return it->second;
     }
-    const DensePlan plan = compute_plan(g, cus, key.forced, key.px_mode);
+    const DensePlan plan = compute_plan(g, cus, key.forced, key.px_mode, device_clock_hz());
     std::lock_guard<std::mutex> lock(mu);
     if (cache.size() >= 4096)
         cache.clear();
@@ -528,7 +556,8 @@ struct PreparedDense {
 // floats, or bytes for the codes entry point), and every kernel then sees a dense, unpadded stride-1 layer with a
 // quarter (stride 2) of the pixels to quantize and sum.  allow_subsample = false keeps the layer as given (callers
 // with their own padding origin).
-int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_subsample = true, int element_bytes = 4)
+int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_subsample = true, int element_bytes = 4,
+                  int px_mode = kPxModeGlobal)
 {
     const bool allow_flat = allow_subsample;   // both are for callers that leave the padding origin to the library
     int rc = geometry(desc, &pd->dims);
@@ -575,7 +604,7 @@ int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_sub
             pd->gk.C4 = quads;
         }
     }
-    pd->plan = make_plan(pd->gk, device_cus());
+    pd->plan = make_plan(pd->gk, device_cus(), px_mode);
     pd->ws = dense_workspace(pd->g, pd->plan, sub_bytes, pd->flat_row_bytes);
     return AXC_OK;
 }
@@ -601,6 +630,15 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
         return rc;
     if (pd.empty)
         return AXC_OK;
+    if (pd.plan.px && workspace_bytes < pd.ws.total) {
+        // No room for the pre-expanded rows: the layer runs the kernel that expands inside its tiles, with the tile
+        // shape and K split the planner prices for THAT kernel, if the workspace holds what that plan needs (its K
+        // split may ask for partial sums the other plan has none of); otherwise with the plan at hand.
+        PreparedDense alt;
+        rc = prepare_dense(desc, &alt, pad_before_override == nullptr, codes_mode ? 1 : 4, -1);
+        if (rc == AXC_OK && workspace_bytes >= alt.ws.total)
+            pd = alt;
+    }
     if (pad_before_override) { // a caller with its own padding rule (tf1 AxConv2D); the plan does not depend on it
         pd.g.ph = pad_before_override[0];
         pd.g.pw = pad_before_override[1];
@@ -1261,10 +1299,19 @@ int axc_conv2d_minmax_static(const axc_table *table, const axc_conv2d_desc *desc
     int rc = prepare_dense(desc, &pd);
     if (rc != AXC_OK)
         return rc;
-    if (pd.ws.total_no_px > kStaticScratchBytes) {
+    size_t needed = pd.plan.px ? pd.ws.total : pd.ws.total_no_px;
+    if (pd.plan.px && needed > kStaticScratchBytes) {
+        // without room for pre-expanded rows the layer runs as run_dense re-plans it, or as planned minus the rows
+        PreparedDense alt;
+        rc = prepare_dense(desc, &alt, true, 4, -1);
+        if (rc != AXC_OK)
+            return rc;
+        needed = std::min(alt.ws.total, pd.ws.total_no_px);
+    }
+    if (needed > kStaticScratchBytes) {
         char msg[200];
         snprintf(msg, sizeof(msg), "layer needs %zu bytes of workspace, the static workspace holds %zu: use "
-                 "axc_conv2d_minmax with a caller-owned workspace", pd.ws.total_no_px, kStaticScratchBytes);
+                 "axc_conv2d_minmax with a caller-owned workspace", needed, kStaticScratchBytes);
         return fail(AXC_INVALID_ARGUMENT, msg);
     }
     void *ws = nullptr;

@@ -181,6 +181,8 @@ inline hipError_t set_max_dynamic_lds_once(const void *kernel, int bytes, bool r
 }
 
 int device_cus();   // compute units of the current device (cached)
+int device_lds_bytes();    // LDS one workgroup may take on the current device (cached)
+double device_clock_hz();  // shader clock of the current device (cached)
 
 // ---- launchers (each enqueues on `stream`; returns hipError_t of the launch) -----------------
 hipError_t launch_quantize_relayout(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,

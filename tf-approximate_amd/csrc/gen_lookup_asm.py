@@ -267,7 +267,7 @@ def emit(nt, buf):
     body_text = " \\\n        ".join(main.lines)
     args = "ACC, ACUR, ANEXT, TAPOFF, CODES, SEL, CHA, CHB, NR, SHIFT, STM, STO, CVO, RD, WR, TAB, WQ, XQ, CSO, QOFF"
     return ("#define PHASE_NT%d_B%d(%s) \\\n    asm volatile( \\\n        %s \\\n"
-            "        : %s \\\n        : %s \\\n        : %s, \"scc\", \"memory\")\n"
+            "        : %s \\\n        : %s \\\n        : %s, \"m0\", \"scc\", \"memory\")\n"
             % (nt, buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))
 
 
@@ -402,7 +402,7 @@ def emit_px(buf):
     body_text = " \\\n        ".join(main.lines)
     args = "ACC, FIRST, SECOND, NFIRST, NSECOND, TAPOFF, SEL, CH, DLF, DLS, L16, NR, STMP, EDST, EOFF, ERC, XQ, QOFF"
     return ("#define PHASE_PX_B%d(%s) \\\n    asm volatile( \\\n        %s \\\n"
-            "        : %s \\\n        : %s \\\n        : %s, \"scc\", \"memory\")\n"
+            "        : %s \\\n        : %s \\\n        : %s, \"m0\", \"scc\", \"memory\")\n"
             % (buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))
 
 

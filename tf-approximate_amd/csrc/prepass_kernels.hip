@@ -1457,7 +1457,7 @@ static bool best_band(const ConvGeom &g, int wseg, int sum_blocks, int64_t lds_l
 {
     const int cus = device_cus();
     const double K = (double)g.KH * g.KW * g.C;
-    const int64_t lds_max = 160 * 1024;
+    const int64_t lds_max = device_lds_bytes();
     const int nsegs = (g.OW + wseg - 1) / wseg;
     const int64_t row_bytes = (int64_t)input_columns_under(g, wseg) * (g.C + 4) * 4;
     bool found = false;
@@ -1493,7 +1493,7 @@ static bool best_band(const ConvGeom &g, int wseg, int sum_blocks, int64_t lds_l
 
 static void choose_band(const ConvGeom &g, int sum_blocks, int *rb_out, int *in_rows_out, int *wseg_out)
 {
-    const int64_t lds_max = 160 * 1024, lds_two = lds_max / 2;
+    const int64_t lds_max = device_lds_bytes(), lds_two = lds_max / 2;
     double t = 0.0;
     int64_t lds = 0;
     *rb_out = 0;
@@ -1652,14 +1652,14 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
             const unsigned grid = (unsigned)(fw.sum8 + work_blocks + fw.pack_blocks);
             if (segmented) {
                 const hipError_t e =
-                    set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_segments_kernel), 160 * 1024);
+                    set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_segments_kernel), device_lds_bytes());
                 if (e != hipSuccess)
                     return e;
                 hipLaunchKernelGGL(patch_sums_segments_kernel, dim3(grid), dim3(block_threads), lds, stream, x, g, rb, in_rows, threads, wseg, tq, lq_dev, psum,
                                    fuse ? xq_fused : nullptr, fw);
                 return hipGetLastError();
             }
-            const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_rows_kernel), 160 * 1024);
+            const hipError_t e = set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_rows_kernel), device_lds_bytes());
             if (e != hipSuccess)
                 return e;
             hipLaunchKernelGGL(patch_sums_rows_kernel, dim3(grid), dim3(block_threads),
