@@ -140,8 +140,9 @@ int axc_qint32_range_for_multiplication(float min_a, float max_a, float min_b, f
 /* How the dense kernel would cut this layer on the current device (for tools and tests; the reference has no
  * counterpart, its launch shapes are fixed in cuda/approx_nn_conv_kernels.cu:296-627):
  * plan = { columns per tile (16/32/64), rows per tile, row tiles, column tiles, K splits, workgroups,
- *          fills of 64 filter entries per K split, 1 if the layer runs out of pre-expanded rows (given a workspace of
- *          the size axc_conv2d_workspace_bytes reports) else 0 }. */
+ *          fills of 64 filter entries per K split, how the layer runs given a workspace of the size
+ *          axc_conv2d_workspace_bytes reports: 0 = table rows expanded inside every tile, 1 = out of pre-expanded
+ *          rows, 2 = out of pre-expanded rows by the kernel whose wavefronts do not meet at a barrier between fills }. */
 int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[8]);
 /* Pins the tile width the planner uses (16, 32 or 64 columns; 0 = its own choice, the default), process-wide, for
  * tests and timing of the wider-tile kernel variants.  The environment variable AXC_TILE_COLUMNS gives the initial
@@ -157,6 +158,13 @@ int axc_set_tile_columns(int columns);
  * plan of the kernel that expands inside its tiles when the workspace holds what that plan needs.  No counterpart
  * in the reference. */
 int axc_set_preexpand(int mode);
+/* The wavefronts of the kernel that plan code 2 stands for wait for each other by polling counters, every wait a bounded
+ * number of polls (the default, 2^20 of ~150 cycles each, is far beyond any legitimate wait).  A wait that runs out ends
+ * the launch early - every wavefront leaves the kernel, nothing hangs - and the NEXT launch call on that GPU returns
+ * AXC_RUNTIME_ERROR once instead of launching: the earlier launch's output is incomplete.  This sets the number of
+ * polls, process-wide; 0 makes every wait that is not satisfied at once give up (tests of the report).  No counterpart
+ * in the reference. */
+int axc_set_wait_limit(uint32_t polls);
 int axc_depthwise_conv2d_workspace_bytes(const axc_conv2d_desc *desc, size_t *bytes);
 
 /* The op: replaces ApproxConv2DOp::Compute -> LaunchApproxConv2DOp<GPUDevice> and the kernels it

@@ -139,14 +139,15 @@ def test_tile_plans_fit_the_kernels(ops, lib):
     """What the planner hands the LUT-GEMM kernels, over many layers and all pinned modes (the query needs no GPU:
     without one it plans for 256 CUs).  A tile holds at most 8 wavefronts x 2 * 64 / columns pixel slots of 64 pixels,
     the row tiles cover the pixels without an empty one, every K split has fills, and pre-expanded rows only come with
-    16-column tiles, channel quads in pairs and splits of whole pairs of fills."""
+    16-column tiles, channel quads in pairs and splits of whole pairs of fills; plan code 2 (the kernel without barriers
+    between fills) only with tiles of 16 to 63 wavefront-rows."""
     shapes = []
     for n, hw in [(1, 1), (1, 7), (2, 8), (4, 14), (64, 14), (64, 28), (16, 56), (64, 56), (128, 32), (128, 8), (3, 33)]:
         for c, co in [(3, 16), (8, 16), (16, 16), (64, 64), (40, 20), (256, 1024), (512, 128), (128, 130), (2048, 512)]:
             for k in (1, 3):
                 if n * hw * hw * max(c, co) <= 64 * 56 * 56 * 1024 and k * k * c < 32768:
                     shapes.append(((n, hw, hw, c), (k, k, c, co)))
-    seen_px = seen_split = seen_px_split = 0
+    seen_px = seen_free = seen_split = seen_px_split = 0
     try:
         for columns, mode in [(0, 0), (0, 1), (0, -1), (16, 1), (32, 0), (64, 0)]:
             assert lib.axc_set_tile_columns(columns) == 0 and lib.axc_set_preexpand(mode) == 0
@@ -170,12 +171,18 @@ def test_tile_plans_fit_the_kernels(ops, lib):
                     assert pl["column_tiles"] * (fps * ks // 2) * 65536 <= (192 << 20) + ks * 65536, what
                 elif mode == 1 and nt == 16 and xs[3] % 8 == 0:
                     assert pl["column_tiles"] * fs[0] * fs[1] * (xs[3] // 8) * 65536 > 192 << 20, what
-                seen_px += pl["preexpanded_rows"]
+                if pl["preexpanded_rows"] == 2:
+                    # the kernel without barriers keeps its counters in the pixel slot a 64th wavefront-row would
+                    # use, and is only picked for tiles of two wavefront-rows per wavefront and 16 fills or more
+                    assert 16 <= rows // 64 <= 63 and fps // 2 >= (16 if fs[0] * fs[1] > 1 else 32), what
+                assert pl["preexpanded_rows"] in (0, 1, 2), what
+                seen_px += bool(pl["preexpanded_rows"])
+                seen_free += pl["preexpanded_rows"] == 2
                 seen_split += ks > 1
-                seen_px_split += pl["preexpanded_rows"] and ks > 1
+                seen_px_split += bool(pl["preexpanded_rows"]) and ks > 1
     finally:
         assert lib.axc_set_tile_columns(0) == 0 and lib.axc_set_preexpand(0) == 0
-    assert seen_px > 50 and seen_split > 50 and seen_px_split > 5
+    assert seen_px > 50 and seen_split > 50 and seen_px_split > 5 and seen_free > 5
 
 
 def test_workspace_sizes(ops, lib):

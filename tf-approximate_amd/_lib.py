@@ -57,6 +57,7 @@ SYMBOLS = [
     ("axc_conv2d_tile_plan", ctypes.c_int, [_desc, ctypes.POINTER(ctypes.c_int32)]),
     ("axc_set_tile_columns", ctypes.c_int, [ctypes.c_int]),
     ("axc_set_preexpand", ctypes.c_int, [ctypes.c_int]),
+    ("axc_set_wait_limit", ctypes.c_int, [ctypes.c_uint32]),
     ("axc_depthwise_conv2d_workspace_bytes", ctypes.c_int, [_desc, ctypes.POINTER(_sz)]),
     ("axc_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),
     ("axc_depthwise_conv2d_minmax", ctypes.c_int, [_vp, _desc, _vp, _vp] + _launch_tail),

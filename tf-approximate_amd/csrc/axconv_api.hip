@@ -119,6 +119,63 @@ int static_scratch(void **ptr)
     return AXC_OK;
 }
 
+// ---- the word through which a LUT-GEMM launch reports a wait between its wavefronts that ran out ----
+// Host memory the device can write, one word per GPU, allocated when the first table is created on that GPU (a launch
+// call allocates nothing).  A launch call that finds the word set reports the failure - of an EARLIER launch on that
+// GPU, whose output is incomplete - clears it and does nothing else.
+std::mutex g_wait_mutex;
+uint32_t *g_wait_host[kMaxDevices] = {};
+uint32_t *g_wait_dev[kMaxDevices] = {};
+std::atomic<uint32_t> g_wait_limit{1u << 20};   // polls per wait, ~150 cycles each: far beyond any fill or epilogue
+
+int wait_error_alloc()
+{
+    int dev = 0;
+    AXC_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices)
+        return AXC_OK;   // launches on such a device run without the report
+    std::lock_guard<std::mutex> lock(g_wait_mutex);
+    if (g_wait_host[dev])
+        return AXC_OK;
+    void *host = nullptr, *devp = nullptr;
+    AXC_HIP(hipHostMalloc(&host, 64, hipHostMallocMapped));
+    memset(host, 0, 64);
+    const hipError_t e = hipHostGetDevicePointer(&devp, host, 0);
+    if (e != hipSuccess) {
+        (void)hipHostFree(host);
+        return fail_hip(e, "hipHostGetDevicePointer");
+    }
+    g_wait_host[dev] = static_cast<uint32_t *>(host);
+    g_wait_dev[dev] = static_cast<uint32_t *>(devp);
+    return AXC_OK;
+}
+
+// The device's view of the word (null if there is none), after reporting what an earlier launch left in it.
+int wait_error_check(uint32_t **dev_word)
+{
+    *dev_word = nullptr;
+    int dev = 0;
+    AXC_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices)
+        return AXC_OK;
+    uint32_t *host = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_wait_mutex);
+        host = g_wait_host[dev];
+        *dev_word = g_wait_dev[dev];
+    }
+    if (!host)
+        return AXC_OK;
+    const uint32_t code = __atomic_exchange_n(host, 0u, __ATOMIC_RELAXED);
+    if (code != 0u) {
+        char msg[200];
+        snprintf(msg, sizeof(msg), "an earlier LUT-GEMM launch on this device gave up a wait between its wavefronts "
+                 "(code %u): its output is incomplete", code);
+        return fail(AXC_RUNTIME_ERROR, msg);
+    }
+    return AXC_OK;
+}
+
 // ---- profiling: events around each kernel, on the launch stream ----
 struct ProfEntry {
     std::vector<std::pair<hipEvent_t, hipEvent_t>> pending;
@@ -624,6 +681,9 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     if (activation != AXC_ACT_NONE && activation != AXC_ACT_RELU)
         return fail(AXC_INVALID_ARGUMENT, "unknown activation");
     const bool codes_mode = input_codes != nullptr;
+    uint32_t *wait_word = nullptr;
+    if (int rc_wait = wait_error_check(&wait_word))
+        return rc_wait;
     PreparedDense pd;
     int rc = prepare_dense(desc, &pd, pad_before_override == nullptr, codes_mode ? 1 : 4);
     if (rc != AXC_OK)
@@ -765,6 +825,8 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     }
     p.px_rows = nullptr;
     p.px_bytes = 0;
+    p.spin_limit = g_wait_limit.load(std::memory_order_relaxed);
+    p.wait_error = wait_word;
     if (use_px) {
         ProfScope ps("px_expand_rows", stream);
         uint16_t *rows = reinterpret_cast<uint16_t *>(ws + pd.ws.px_off);
@@ -982,6 +1044,7 @@ int axc_table_create(const uint16_t *host_table, axc_table **out)
     // device image); a failure here is reported by axc_conv2d_minmax_static, which looks again
     void *unused = nullptr;
     (void)static_scratch(&unused);
+    (void)wait_error_alloc();   // without the word, launches run with no report of a wait that ran out
     *out = tab;
     return AXC_OK;
 }
@@ -1216,7 +1279,13 @@ int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[8])
     plan[4] = pd.plan.k_splits;
     plan[5] = pd.plan.grid;
     plan[6] = pd.plan.k_splits > 1 ? pd.plan.fills_per_split : pd.plan.fills;
-    plan[7] = pd.plan.px;
+    plan[7] = pd.plan.px ? (px_free_running(pd.plan, pd.gk.KH * pd.gk.KW) ? 2 : 1) : 0;
+    return AXC_OK;
+}
+
+int axc_set_wait_limit(uint32_t polls)
+{
+    g_wait_limit.store(polls, std::memory_order_relaxed);
     return AXC_OK;
 }
 

@@ -20,6 +20,8 @@ constexpr int kDenseLdsBytes = 4 * kExpandBytes; // dense kernel: 2 buffers of e
 constexpr int kDenseThreads = 512;             // dense kernel: 8 wavefronts x 256 VGPRs, one workgroup per CU
 constexpr int kDenseWaves = kDenseThreads / 64;
 constexpr int kDenseParkBytes = 16 * 4 * kDenseThreads; // per-thread pixel geometry parked behind the buffers
+constexpr int kPxMaxTileWaveRows = 8 * kDenseWaves - 1;  // lutgemm_pxf_kernel: the last wavefront's last pixel slot holds
+                                                         // the kernel's wait counters instead of geometry
 constexpr int kBlockThreads = 1024;            // depthwise kernel / LDS probe: 16 wavefronts per CU
 constexpr int kWaves = kBlockThreads / 64;
 // Accumulate instruction mix of the dense kernel's generated phase body (gen_lookup_asm.py emits the same):
@@ -114,6 +116,11 @@ struct DenseParams {
     uint32_t quad_bytes;         // between the channel quads that one tap of a pixel reads
     uint32_t zp_tail_bytes;      // size of the zero-point row behind xq
     int flat_col_bytes;          // flat: bytes between horizontally neighbouring output pixels (sw * C); 0 = usual layout
+    // lutgemm_pxf_kernel: its wavefronts wait for each other through counters in LDS, every wait a bounded number of
+    // polls.  A wait that runs out writes a nonzero word to *wait_error (host-visible memory) and the wavefront leaves
+    // the kernel; so do the others at their next wait.
+    uint32_t spin_limit;
+    uint32_t *wait_error;
 };
 
 struct DepthwiseParams {
@@ -227,6 +234,7 @@ hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream);
 hipError_t launch_px_expand_rows(const uint16_t *wq, const uint16_t *tableT, const DensePlan &plan, uint16_t *rows,
                                  hipStream_t stream);
 hipError_t launch_dense_px(const DenseParams &p, bool out_i32, hipStream_t stream);
+bool px_free_running(const DensePlan &plan, int taps);   // the plan runs lutgemm_pxf_kernel (no barrier between fills)
 hipError_t launch_splitk_epilogue(const DenseParams &p, const int32_t *partials, float *out_f, int32_t *out_i,
                                   hipStream_t stream);
 hipError_t launch_axconv_correction(const uint8_t *codes, const uint8_t *fcodes, const ConvGeom &g, int offset_input,

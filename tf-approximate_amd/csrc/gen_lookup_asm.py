@@ -406,6 +406,219 @@ def emit_px(buf):
             % (buf, args, body_text, ", ".join(outs), ", ".join(inp), clob))
 
 
+# LDS control block of the kernel that reads pre-expanded fills: the last 32 bytes of the 160 KiB (the geometry slots
+# of a wavefront-row that its tiles never have).  One counter per fill buffer that only grows: the eight wavefronts
+# count themselves (one lane adds 1) when their share of a fill has arrived in the buffer, and again when they have
+# finished reading that fill.  All eight arrivals of a fill precede the first reader, and all eight readers the
+# first arrival of the next fill, so the j-th fill of a buffer is whole once the count has reached 16 j + 8 and
+# the buffer free again at 16 j + 16.  EVENTS[0], EVENTS[1], ABORT.
+PX_LDS_BYTES = 163840
+PX_CB = PX_LDS_BYTES - 32
+PX_TGT_ISSUED = 0xfffffffe     # TGT of a phase that has issued its loads,
+PX_TGT_COUNTED = 0xffffffff    # and of one that has also counted their arrival
+IB_STS_VM_CNT = 0x00c0000f     # the bits of the hardware register IB_STS that hold this wavefront's vmcnt
+PX_FIRST = ADDR_BASE - 2       # first register the phase of the pre-expanded kernel clobbers
+SCRATCH_ADDR = PX_FIRST        # address temporary of the activation loads, the polls and the count
+POLL_REG = PX_FIRST + 1        # where a poll lands: EVENTS[other]
+
+
+def emit_pxf():
+    """PHASE_PXF: one phase of the kernel variant that reads pre-expanded fills WITHOUT a barrier between fills.
+
+    A fill here is a pair of ordinary fills: 8 input channels x 16 columns = 128 slots, so that the expanded row of
+    an activation code is 256 bytes, one pass over all 64 LDS banks.  The rows of a fill are built once per layer
+    in memory and every wavefront copies its eighth of the next fill (eight buffer loads with the lds modifier)
+    straight into the other LDS buffer.  A lane owns two activation dwords per pixel and fill, FIRST
+    and SECOND; lanes with bit 3 set hold the two swapped, and read FIRST out of the upper half of the row, so that
+    the 16 lanes that share an LDS pass read 16 different 16-byte chunks.  A pixel is looked up as two units of
+    eight steps (FIRST, then SECOND) that run through the same rolling window of eight reads.
+
+    The wavefronts of a workgroup do not meet at a barrier between fills.  The other buffer may be refilled once
+    all eight wavefronts have finished the fill before this one: the phase polls EVENTS[other] when
+    it starts on a pixel (one 4-byte LDS read, consumed a unit later, where the waits for the lookups have long
+    covered it).  TGT carries the state.  Below 0xfffffffd it is the count EVENTS[other] has to reach: the first poll
+    that finds it there issues the eight loads and sets TGT to 0xfffffffe (the caller does the same when it finds
+    the buffer free before the phase).  From there every poll looks, without waiting, whether this wavefront still
+    has a load in flight (its vmcnt, read from the hardware register IB_STS): the first poll that finds none adds
+    the wavefront to EVENTS[other] and sets TGT to 0xffffffff.  A wavefront never waits for the loads inside the
+    phase: a fill takes some 3 000 cycles to land under the lookups.  A
+    phase that ends with TGT below 0xffffffff leaves what is missing to the caller.  SEEN returns the last
+    EVENTS[other] a poll saw (0 without a poll): the caller may start on the next fill without a look of its own.
+
+    One body serves both buffers.  The lookup address (buffer << 16 | row << 8 | half << 7 | chunk << 4) is one
+    v_perm_b32: byte 2 <- byte 3 of the chunk register (0 or 1: the caller flips it between phases), byte 1 <- the
+    activation code, byte 0 <- one of the three chunk bytes the register holds (steps 0-2, 3-5, 6-7 of a unit).  The
+    LDS destination of the loads (EDST: the wavefront's eighth of the OTHER buffer) and the address of the counter
+    the polls read (POLLADDR: DONE of the other buffer) are scalar operands.
+    """
+    rows = 8
+
+    def address(st, r, h, step):
+        va = ADDR_BASE + (step % 4)
+        st.ins("v_perm_b32 v%d, %%[%s%d], %%[ch%d%s], %%[s%d]" % (va, "fg"[h], r, h, "abc"[step // 3], step))
+
+    def read(st, r, h, step, with_address=True):
+        b = TEMP_BASE + 4 * step
+        va = ADDR_BASE + (step % 4)
+        if with_address:
+            address(st, r, h, step)
+        return st.lds("ds_read_b128 v[%d:%d], v%d" % (b, b + 3, va))
+
+    def adds(st, r, steps, halfway=None):
+        """Twelve adds; no instruction reads the result of the one right before it."""
+        g = steps[0] % 2
+        sdwa = "v_add_u32_sdwa %s, %s, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
+        even = lambda d: "%%[c%d_%d]" % (r, g * 8 + 2 * d)
+        odd = lambda d: "%%[c%d_%d]" % (r, g * 8 + 2 * d + 1)
+        reg = lambda k, d: TEMP_BASE + 4 * steps[k] + d
+        for pair in ((0, 1), (2, 3)):
+            if pair[0] == 2 and halfway:
+                halfway()
+            for d in pair:
+                st.ins("v_add3_u32 %s, %s, v%d, v%d" % (even(d), even(d), reg(0, d), reg(1, d)))
+            for k in range(2):
+                for d in pair:
+                    st.ins(sdwa % (odd(d), odd(d), reg(k, d)))
+
+    groups = [(0, 2), (1, 3), (4, 6), (5, 7)]
+    counter = [0]
+
+    def fresh(prefix):
+        counter[0] += 1
+        return "%s%d_%%=" % (prefix, counter[0])
+
+    def poll_issue(st, state):
+        st.ins("v_mov_b32 v%d, %%[polladdr]" % SCRATCH_ADDR)
+        state["poll"] = st.lds("ds_read_b32 v%d, v%d" % (POLL_REG, SCRATCH_ADDR))
+
+    def poll_consume(st, state):
+        st.wait(state["poll"])
+        issued, end = fresh("Lis"), fresh("Lpe")
+        st.ins("v_readfirstlane_b32 %%[seen], v%d" % POLL_REG)
+        st.ins("s_cmp_ge_u32 %%[tgt], 0x%x" % PX_TGT_ISSUED)
+        st.ins("s_cbranch_scc1 %s" % issued)
+        # not yet issued: if all eight wavefronts have left the other buffer, the eight loads of 1 KiB, memory -> LDS
+        st.ins("s_cmp_ge_u32 %[seen], %[tgt]")
+        st.ins("s_cbranch_scc0 %s" % end)
+        for j in range(8):
+            st.ins("s_add_u32 m0, %%[edst], %d" % (j * 1024))
+            st.ins("s_add_u32 %%[stmp], %%[eoff], %d" % (j * 1024))
+            st.ins("buffer_load_dwordx4 %[l16], %[erc], %[stmp] offen lds")
+            st.ins("s_nop 0")
+        st.ins("s_mov_b32 %%[tgt], 0x%x" % PX_TGT_ISSUED)
+        st.ins("s_branch %s" % end)
+        st.label(issued)
+        # issued: once none of this wavefront's loads is in flight any more, add it to EVENTS[other]
+        st.ins("s_cmp_eq_u32 %[tgt], -1")
+        st.ins("s_cbranch_scc1 %s" % end)
+        st.ins("s_getreg_b32 %[stmp], hwreg(HW_REG_IB_STS)")
+        st.ins("s_and_b32 %%[stmp], %%[stmp], 0x%x" % IB_STS_VM_CNT)
+        st.ins("s_cbranch_scc1 %s" % end)
+        st.ins("v_mov_b32 v%d, %%[polladdr]" % SCRATCH_ADDR)
+        st.ins("v_mov_b32 v%d, 1" % POLL_REG)
+        st.ins("s_mov_b64 %[sx], exec")          # one lane adds: 64 atomics on one address would hold the LDS for as many turns
+        st.ins("s_mov_b64 exec, 1")
+        st.ins("ds_add_u32 v%d, v%d" % (SCRATCH_ADDR, POLL_REG))   # not in the model's queue: waits stay on the safe side
+        st.ins("s_mov_b64 exec, %[sx]")
+        st.ins("s_mov_b32 %[tgt], -1")
+        st.label(end)
+
+    def act_load(r):         # both activation dwords of pixel r for the next fill; skipped for a pixel the wavefront
+        def f(st, state):    # does not have (a gather costs the CU's address unit as much as 1 KiB of the fill)
+            label = None
+            if r > 0:
+                label = fresh("Lskip")
+                st.ins("s_cmp_lt_u32 %d, %%[nr]" % r)
+                st.ins("s_cbranch_scc0 %s" % label)
+            st.ins("v_add_u32 v%d, %%[t%d], %%[dlf]" % (SCRATCH_ADDR, r))
+            st.ins("buffer_load_dword %%[nf%d], v%d, %%[xq], %%[qoff] offen" % (r, SCRATCH_ADDR))
+            st.ins("v_add_u32 v%d, %%[t%d], %%[dls]" % (SCRATCH_ADDR, r))
+            st.ins("buffer_load_dword %%[ng%d], v%d, %%[xq], %%[qoff] offen" % (r, SCRATCH_ADDR))
+            if label:
+                st.label(label)
+        return f
+
+    aux = [act_load(r) for r in range(rows)]
+
+    def aux_step(st, state):
+        if state["pos"] < len(aux):
+            aux[state["pos"]](st, state)
+            state["pos"] += 1
+
+    def aux_rest(st, state):
+        while state["pos"] < len(aux):
+            aux_step(st, state)
+
+    def body(st, u, pending, with_next, state):
+        """Accumulate unit u = 2 * pixel + half; with_next: refill the window with unit u + 1."""
+        r, nxt = u // 2, [None] * 8
+        for gi, steps in enumerate(groups):
+            st.wait(max((pending[s] for s in steps), key=lambda op: st.fifo.index(op) if op in st.fifo else -1))
+            # the addresses of the next two lookups are computed in the middle of the adds, well ahead of the reads
+            # that use them: a read right behind its v_perm_b32 waits for that instruction's result
+            early = (lambda: [address(st, (u + 1) // 2, (u + 1) % 2, s) for s in steps]) if with_next else None
+            adds(st, r, steps, early)
+            if u % 2 == 1 and gi == 1:
+                poll_consume(st, state)
+            for s in steps:
+                if with_next:
+                    nxt[s] = read(st, (u + 1) // 2, (u + 1) % 2, s, with_address=False)
+                aux_step(st, state)
+            if u % 2 == 0 and gi == 0:
+                poll_issue(st, state)
+        return nxt
+
+    main = Stream()
+    main.ins("s_mov_b32 %[seen], 0")
+    main.ins("s_cmp_eq_u32 %[nr], 0")
+    main.ins("s_cbranch_scc1 Lzero_%=")
+    pending = [read(main, 0, 0, s) for s in range(8)]
+    state = {"pos": 0, "poll": None}
+    forks = []
+    for r in range(rows):
+        pending = body(main, 2 * r, pending, True, state)
+        if r < rows - 1:
+            main.ins("s_cmp_lt_u32 %d, %%[nr]" % (r + 1))
+            main.ins("s_cbranch_scc0 Llast%d_%%=" % r)
+            forks.append((r, main.fork(), list(pending), dict(state)))
+            pending = body(main, 2 * r + 1, pending, True, state)
+        else:
+            body(main, 2 * r + 1, pending, False, state)
+    aux_rest(main, state)
+    main.drain()
+    main.ins("s_branch Lend_%=")
+    for r, st, pend, stt in forks:
+        st.label("Llast%d_%%=" % r)
+        body(st, 2 * r + 1, pend, False, stt)
+        aux_rest(st, stt)
+        st.drain()
+        st.ins("s_branch Lend_%=")
+    zero = Stream(main.lines)
+    zero.label("Lzero_%=")
+    aux_rest(zero, {"pos": 0, "poll": None})
+    zero.drain()
+    zero.label("Lend_%=")
+
+    outs = ['[c%d_%d] "+v"(ACC[%d][%d])' % (r, i, r, i) for r in range(rows) for i in range(16)]
+    outs += ['[nf%d] "=&v"(NFIRST[%d])' % (r, r) for r in range(rows)]
+    outs += ['[ng%d] "=&v"(NSECOND[%d])' % (r, r) for r in range(rows)]
+    outs += ['[stmp] "=&s"(STMP)', '[tgt] "+s"(TGT)', '[seen] "=&s"(SEEN)', '[sx] "=&s"(SX)']
+    inp = ['[f%d] "v"(FIRST[%d])' % (r, r) for r in range(rows)]
+    inp += ['[g%d] "v"(SECOND[%d])' % (r, r) for r in range(rows)]
+    inp += ['[t%d] "v"(TAPOFF[%d])' % (r, r) for r in range(rows)]
+    inp += ['[s%d] "v"(SEL[%d])' % (i, i) for i in range(8)]
+    inp += ['[ch%d%s] "v"(CH[%d])' % (h, "abc"[i], 3 * h + i) for h in range(2) for i in range(3)]
+    inp += ['[dlf] "v"(DLF)', '[dls] "v"(DLS)', '[l16] "v"(L16)', '[nr] "s"(NR)', '[polladdr] "s"(POLLADDR)']
+    inp += ['[edst] "s"(EDST)', '[eoff] "s"(EOFF)', '[erc] "s"(ERC)', '[xq] "s"(XQ)', '[qoff] "s"(QOFF)']
+    clob = ", ".join('"v%d"' % r for r in range(PX_FIRST, TEMP_BASE + 32))
+    body_text = " \\\n        ".join(main.lines)
+    args = ("ACC, FIRST, SECOND, NFIRST, NSECOND, TAPOFF, SEL, CH, DLF, DLS, L16, NR, STMP, SX, TGT, SEEN, POLLADDR, EDST, "
+            "EOFF, ERC, XQ, QOFF")
+    return ("#define PHASE_PXF(%s) \\\n    asm volatile( \\\n        %s \\\n"
+            "        : %s \\\n        : %s \\\n        : %s, \"m0\", \"scc\", \"memory\")\n"
+            % (args, body_text, ", ".join(outs), ", ".join(inp), clob))
+
+
 if __name__ == "__main__":
     print("// Generated by gen_lookup_asm.py -- do not edit.")
     for nt in (16, 32, 64):
@@ -413,3 +626,4 @@ if __name__ == "__main__":
             print(emit(nt, buf))
     for buf in (0, 1):
         print(emit_px(buf))
+    print(emit_pxf())

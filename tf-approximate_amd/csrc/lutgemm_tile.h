@@ -32,7 +32,9 @@ struct TileRows {
     int64_t wr_end;         // end of the pixels owned by this wavefront's half
     int wr_base;
 };
-template <int R, bool EVEN_SMALL = false>
+// ROUND_ROBIN: wavefront-row i goes to SIMD i & 3 whichever half owns it (wavefront w sits on SIMD w & 3), so the
+// SIMDs' loads differ by one row at most however the rows divide between the halves.
+template <int R, bool EVEN_SMALL = false, bool ROUND_ROBIN = false>
 __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, int wave)
 {
     TileRows t;
@@ -47,7 +49,7 @@ __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, i
     wr_old = wr_old > 4 * R ? 4 * R : wr_old;
     wr_old = wr_old < wrows - 4 * R ? wrows - 4 * R : wr_old;
     const bool old_half = wave < kDenseWaves / 2;
-    t.wr_base = old_half ? wave : wr_old + wave - kDenseWaves / 2;
+    t.wr_base = old_half ? wave : wr_old + (ROUND_ROBIN ? ((wave - wr_old) & 3) : wave - kDenseWaves / 2);
     t.wr_end = t.row0 + (int64_t)(old_half ? wr_old : wrows) * 64;
     return t;
 }
@@ -57,8 +59,11 @@ __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, i
 // quad 0 in address units (may point outside the image), slot 2r+1 = input coordinates of tap (0, 0) as (ih0 << 16) | (iw0 & 0xffff),
 // 0x80000000 for a pixel that does not exist.  Returns the number of this lane's pixels whose wavefront-row exists
 // (a prefix of the R; the same in every lane of the wavefront).
-template <int R>
-__device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const TileRows &t, int lane, uint32_t *park)
+// STRIDE: dwords between a thread's slots (kDenseThreads: slot-major over the workgroup; 64: every wavefront owns a
+// contiguous piece).  skip_row: a pixel slot that is not written (its place in LDS belongs to something else).
+template <int R, int STRIDE = kDenseThreads>
+__device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const TileRows &t, int lane, uint32_t *park,
+                                                  const int skip_row = -1)
 {
     const ConvGeom &g = p.g;
     const int rowstep = p.row_step;
@@ -90,8 +95,10 @@ __device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const Ti
         // and never outside (stored as column 0)
         const int ih0 = oh * g.sh - g.ph, iw0 = p.flat_col_bytes ? 0 : ow * g.sw - g.pw;
         const int col = p.flat_col_bytes ? ow * p.flat_col_bytes : iw0;
-        park[(2 * r) * kDenseThreads] = valid ? (uint32_t)((n * g.H + ih0) * rowstep + col) : 0u;
-        park[(2 * r + 1) * kDenseThreads] = valid ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
+        if (r != skip_row) {
+            park[(2 * r) * STRIDE] = valid ? (uint32_t)((n * g.H + ih0) * rowstep + col) : 0u;
+            park[(2 * r + 1) * STRIDE] = valid ? (uint32_t)((ih0 << 16) | (iw0 & 0xffff)) : 0x80000000u;
+        }
         // the next pixel of this lane: p.step_* = (n, oh, ow) of 64 * kDenseWaves / 2 output pixels
         ow += p.step_ow;
         const int c1 = ow >= g.OW ? 1 : 0;
@@ -106,7 +113,7 @@ __device__ __forceinline__ uint32_t park_geometry(const DenseParams &p, const Ti
 
 // byte offset in xq of quad 0 of tap (kh, kw) for each of the lane's pixels; the zero-point row outside the image.
 // live (the same for the whole wavefront): only the first `live` pixels are recomputed, the others keep what they hold.
-template <int R>
+template <int R, int STRIDE = kDenseThreads>
 __device__ __forceinline__ void tap_offsets(const DenseParams &p, const uint32_t *park, int kh, int kw, uint32_t zp_row,
                                             uint32_t (&idx_tap)[R], uint32_t live = R)
 {
@@ -117,8 +124,8 @@ __device__ __forceinline__ void tap_offsets(const DenseParams &p, const uint32_t
     for (int r = 0; r < R; ++r) {
         if ((uint32_t)r >= live)
             break;
-        const int32_t pb = (int32_t)park[(2 * r) * kDenseThreads];
-        const int32_t hw = (int32_t)park[(2 * r + 1) * kDenseThreads];
+        const int32_t pb = (int32_t)park[(2 * r) * STRIDE];
+        const int32_t hw = (int32_t)park[(2 * r + 1) * STRIDE];
         const int ih = (hw >> 16) + dh;
         const int iw = (int)(int16_t)(hw & 0xffff) + dw;
         const bool inb = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
@@ -150,7 +157,10 @@ __device__ __forceinline__ void fix_even_columns(int32_t (&acc)[R][NT])
 // 64-byte pieces of memory.  With NT <= 32 and Co % 4 == 0 the wavefront therefore turns each of its wavefront-rows
 // through a private piece of LDS (turn + wave * 64 * (NT * 4 + 16) bytes; the caller guarantees that nothing else
 // uses it) so that NT/4 neighbouring lanes write one pixel's NT columns: 16 or 8 contiguous runs per store.
-template <int NT, bool OUT_I32>
+//
+// HALF_TURN: `turn` is the wavefront's own piece already, and only 32 * (NT * 4 + 16) bytes of it: a wavefront-row
+// goes through it as two halves of 32 pixels.
+template <int NT, bool OUT_I32, bool HALF_TURN = false>
 __device__ __forceinline__ void store_tile(const DenseParams &p, int32_t (&acc)[2 * (64 / NT)][NT], const TileRows &t,
                                            const int ct, const int ksi, const uint32_t nr_s, const int lane,
                                            const int wave, unsigned char *const turn)
@@ -181,7 +191,7 @@ __device__ __forceinline__ void store_tile(const DenseParams &p, int32_t (&acc)[
     if (kTransposed && (g.Co & 3) == 0) {
         constexpr int Q = NT / 4;                 // 16-byte quads (lanes) per pixel
         constexpr int PITCH = NT * 4 + 16;        // bytes per pixel in LDS: the +16 spreads pixels over the banks
-        unsigned char *const wl = turn + (size_t)wave * 64 * PITCH;
+        unsigned char *const wl = HALF_TURN ? turn : turn + (size_t)wave * 64 * PITCH;
         typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
         // Behind the transposition a lane stores the same four columns of every pixel it handles: the terms
         // that depend on the column (filter sum, bias) are applied there, from four registers each.
@@ -204,43 +214,50 @@ __device__ __forceinline__ void store_tile(const DenseParams &p, int32_t (&acc)[
                 const int64_t m0 = t.row0 + (int64_t)(t.wr_base + r * (kDenseWaves / 2)) * 64;
                 const int nvalid = (int)(t.row_end - m0 < 64 ? t.row_end - m0 : 64);
                 const float t1 = __fmul_rn(e_m2, ps[r]);
-#pragma unroll
-                for (int set = 0; set < SETS; ++set) {
-                    const int h = (c0 + set) & (SETS - 1);
-                    uint32_t w[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        if (OUT_I32)
-                            w[e] = (uint32_t)acc[r][set * 8 + e];
-                        else
-                            w[e] = __float_as_uint(__fadd_rn(__fmul_rn((float)acc[r][set * 8 + e], e_s1xs2), t1));
-                    }
-                    u32x4s lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
-                    *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32) = lo;
-                    *reinterpret_cast<u32x4s *>(wl + lane * PITCH + h * 32 + 16) = hi;
-                }
                 uint32_t *const out = OUT_I32 ? reinterpret_cast<uint32_t *>(p.out_i) + (int64_t)ksi * g.M * g.Co
                                               : reinterpret_cast<uint32_t *>(p.out_f);
+                constexpr int PASSES = HALF_TURN ? 2 : 1, PIX = 64 / PASSES;   // pixels per pass through LDS
 #pragma unroll
-                for (int i = 0; i < Q; ++i) {
-                    const int pix = i * (64 / Q) + lane / Q;
-                    u32x4s d = *reinterpret_cast<const u32x4s *>(wl + pix * PITCH + quad * 16);
-                    if (!OUT_I32) {
+                for (int pass = 0; pass < PASSES; ++pass) {
+                    if (!HALF_TURN || (lane >> 5) == pass) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            float v = __fsub_rn(__fadd_rn(__uint_as_float(d[j]), t3q[j]), e_km);
-                            if (kBias)
-                                v = __fadd_rn(v, biasq[j]);
-                            d[j] = __float_as_uint(kRelu ? fmaxf(v, 0.0f) : v);
+                        for (int set = 0; set < SETS; ++set) {
+                            const int h = (c0 + set) & (SETS - 1);
+                            uint32_t w[8];
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                if (OUT_I32)
+                                    w[e] = (uint32_t)acc[r][set * 8 + e];
+                                else
+                                    w[e] = __float_as_uint(__fadd_rn(__fmul_rn((float)acc[r][set * 8 + e], e_s1xs2), t1));
+                            }
+                            u32x4s lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};
+                            *reinterpret_cast<u32x4s *>(wl + (lane & (PIX - 1)) * PITCH + h * 32) = lo;
+                            *reinterpret_cast<u32x4s *>(wl + (lane & (PIX - 1)) * PITCH + h * 32 + 16) = hi;
                         }
                     }
-                    if (pix < nvalid && colq < g.Co) {
-                        // the float output is not read again by this op: streamed past the caches, which keeps
-                        // them for the activations; split-K partial sums are read back at once and stay cached
-                        if (OUT_I32)
-                            *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq) = d;
-                        else
-                            __builtin_nontemporal_store(d, reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq));
+#pragma unroll
+                    for (int i = 0; i < Q / PASSES; ++i) {
+                        const int pl = i * (64 / Q) + lane / Q;      // pixel within the pass
+                        const int pix = pass * PIX + pl;
+                        u32x4s d = *reinterpret_cast<const u32x4s *>(wl + pl * PITCH + quad * 16);
+                        if (!OUT_I32) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                float v = __fsub_rn(__fadd_rn(__uint_as_float(d[j]), t3q[j]), e_km);
+                                if (kBias)
+                                    v = __fadd_rn(v, biasq[j]);
+                                d[j] = __float_as_uint(kRelu ? fmaxf(v, 0.0f) : v);
+                            }
+                        }
+                        if (pix < nvalid && colq < g.Co) {
+                            // the float output is not read again by this op: streamed past the caches, which keeps
+                            // them for the activations; split-K partial sums are read back at once and stay cached
+                            if (OUT_I32)
+                                *reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq) = d;
+                            else
+                                __builtin_nontemporal_store(d, reinterpret_cast<u32x4s *>(out + (m0 + pix) * g.Co + colq));
+                        }
                     }
                 }
             }

@@ -325,6 +325,8 @@ def conv2d_tile_plan(input_shape, filter_shape, strides=(1, 1, 1, 1), padding="S
     desc = make_desc(tuple(input_shape), tuple(filter_shape), list(strides), padding, (), "NHWC", list(dilations), 8)
     plan = (ctypes.c_int32 * 8)()
     _check(lib.axc_conv2d_tile_plan(ctypes.byref(desc), plan))
+    # preexpanded_rows: 0 = rows expanded inside every tile, 1 = pre-expanded rows, 2 = pre-expanded rows read by the
+    # kernel without a barrier between fills
     keys = ("columns_per_tile", "rows_per_tile", "row_tiles", "column_tiles", "k_splits", "workgroups",
             "fills_per_split", "preexpanded_rows")
     return dict(zip(keys, [int(v) for v in plan]))
@@ -338,6 +340,12 @@ def set_tile_columns(columns):
 def set_preexpand(mode):
     """Which dense layers run out of pre-expanded rows: 0 = the planner's choice, 1 = all that can, -1 = none."""
     _check(_lib.load().axc_set_preexpand(int(mode)))
+
+
+def set_wait_limit(polls):
+    """Polls a wavefront of the barrier-free LUT-GEMM kernel makes in one wait before it gives up (tests of the
+    report; the default is 2**20)."""
+    _check(_lib.load().axc_set_wait_limit(int(polls)))
 
 
 _table_cache = {}
