@@ -46,6 +46,8 @@ WORKLOADS = {
     "dw3x3_b64_112x112x192_s1": ((64, 112, 112, 192), (3, 3, 192, 1), (1, 1), True),
     "dw3x3_b64_112x112x192_s2": ((64, 112, 112, 192), (3, 3, 192, 1), (2, 2), True),
     "conv3x3_b128_32x32x16_to_16": ((128, 32, 32, 16), (3, 3, 16, 16), (1, 1), False),
+    "conv3x3_b64_28x28x128_to_128": ((64, 28, 28, 128), (3, 3, 128, 128), (1, 1), False),   # K cut in two, pre-expanded rows
+    "conv3x3_b64_7x7x512_to_512": ((64, 7, 7, 512), (3, 3, 512, 512), (1, 1), False),       # K cut over tiles, rows expanded in the tiles
 }
 DEFAULT = "conv3x3_b64_56x56x64_to_64_s1_same"
 
@@ -80,22 +82,28 @@ CPU_SAMPLE_S = 0.5      # single-thread reference sample per `layers` record
 # device copy of known size inside the same run.  Keyed by (workload, kernel); not measured in the run that prints
 # them: the bench line says which profile they come from.
 PROFILED_TRAFFIC = {
-    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 80848.9 * 1024 + 1.000 * 62076.4 * 1024,
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 81240.4 * 1024 + 1.000 * 64616.7 * 1024,
                                                            "profiles/lutgemm_px_conv3x3_b64_56x56x64.md"),
-    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8312.5 * 1024 + 1.000 * 61757.9 * 1024,
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8312.5 * 1024 + 1.000 * 62356.2 * 1024,
                                                                "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
-    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48275.5 * 1024 + 1.000 * 784460.2 * 1024,
+    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48254.9 * 1024 + 1.000 * 790653.1 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b64_112x112x32_to_192.md"),
-    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37242.1 * 1024 + 1.000 * 262539.4 * 1024,
+    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37246.2 * 1024 + 1.000 * 266142.7 * 1024,
                                                     "profiles/lutgemm_px_conv1x1_b64_56x56x64_to_256.md"),
-    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 466401.4 * 1024 + 1.000 * 503985.5 * 1024,
+    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 471020.5 * 1024 + 1.000 * 469768.6 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
-    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 92846.3 * 1024 + 1.000 * 272367.6 * 1024,
+    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 94017.3 * 1024 + 1.000 * 244659.8 * 1024,
                                                       "profiles/lutgemm_px_conv7x7s2_b64_224x224x3_to_64.md"),
-    ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51701.5 * 1024 + 1.000 * 106261.2 * 1024,
+    ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51701.8 * 1024 + 1.000 * 106354.8 * 1024,
                                                          "profiles/lutgemm_expand_conv3x3_b64_28x28x512_to_512.md"),
-    ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6128.5 * 1024 + 1.025 * 8192.0 * 1024,
+    ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6109.0 * 1024 + 1.025 * 8192.0 * 1024,
                                                     "profiles/lutgemm_px_conv3x3_b128_32x32x16_to_16.md"),
+    ("conv1x1_b64_112x112x192_to_32", "lutgemm_px"): (2.000 * 101813.4 * 1024 + 1.000 * 129282.3 * 1024,
+                                                      "profiles/lutgemm_px_conv1x1_b64_112x112x192_to_32.md"),
+    ("conv3x3_b64_28x28x128_to_128", "lutgemm_px"): (2.000 * 130200.1 * 1024 + 1.000 * 54405.0 * 1024,
+                                                     "profiles/lutgemm_px_conv3x3_b64_28x28x128_to_128.md"),
+    ("conv3x3_b64_7x7x512_to_512", "lutgemm_expand"): (2.000 * 8872.9 * 1024 + 1.000 * 55096.7 * 1024,
+                                                       "profiles/lutgemm_expand_conv3x3_b64_7x7x512_to_512.md"),
     ("dw3x3_b64_112x112x192_s1", "depthwise_lut"): (2.000 * 342889 * 1024 + 1.000 * 602112 * 1024,
                                                     "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
     ("dw3x3_b64_112x112x192_s2", "depthwise_lut"): (2.000 * 321245 * 1024 + 1.000 * 150528 * 1024,
@@ -354,7 +362,7 @@ def measure_layer(pkg, ops, oracle, ceil, spec, steps=None, preroll_s=0.08):
     return rec
 
 
-def measure_network(pkg, name, steps, warmup, fused_layers=False):
+def measure_network(pkg, name, steps, warmup, fused_layers=False, graph=False):
     import torch
     from tf_approximate_amd import networks
     synth = pkg.synth
@@ -373,12 +381,60 @@ def measure_network(pkg, name, steps, warmup, fused_layers=False):
         net.forward(xin)
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / steps
-    return {"network": name, "input": list(xin.shape), "convolutions": net.conv_count(), "steps": steps,
-            "ms_per_pass": round(ms, 4), "images_per_s": round(xin.shape[0] / (ms * 1e-3), 1),
-            "approx_macs_per_pass": macs, "approx_gmac_per_s": round(macs / (ms * 1e-3) / 1e9, 1),
-            "fused_layers": bool(fused_layers), "layers_not_fused": net.unfused_layers() if fused_layers else [],
-            "note": "convolutions through the op, a ReLU that directly follows one fused into its store; adds (with their ReLU) "
-                    "and the max-pool in torch"}
+    rec = {"network": name, "input": list(xin.shape), "convolutions": net.conv_count(), "steps": steps,
+           "ms_per_pass": round(ms, 4), "images_per_s": round(xin.shape[0] / (ms * 1e-3), 1),
+           "approx_macs_per_pass": macs, "approx_gmac_per_s": round(macs / (ms * 1e-3) / 1e9, 1),
+           "fused_layers": bool(fused_layers), "layers_not_fused": net.unfused_layers() if fused_layers else [],
+           "note": "convolutions through the op, a ReLU that directly follows one fused into its store; adds (with their ReLU) "
+                   "and the max-pool in torch"}
+    if graph:
+        rec["hip_graph"] = graph_replay(net, xin, steps)
+    return rec
+
+
+def graph_replay(net, xin, steps):
+    """The same pass recorded once into a HIP graph and replayed: the library allocates nothing and never waits for the
+    device inside a call, so a whole network is one graph launch and the host's per-call work (about as long as a
+    small layer's kernels) drops out.  Every checked replay must reproduce the eager output bit for bit, with eager
+    passes and synchronizations between the replays.  A failure is reported, not raised: the eager figures stand."""
+    import torch
+    try:
+        want = net.forward(xin)[0].clone()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):      # first calls on the capture stream: its workspace, lazily set attributes
+            for _ in range(2):
+                net.forward(xin)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            out = net.forward(xin)[0]
+        exact = True
+        for _ in range(3):
+            out.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            exact = exact and bool(torch.equal(out, want))
+            net.forward(xin)               # eager work between the replays
+            torch.cuda.synchronize()
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.replay()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        g.replay()
+        torch.cuda.synchronize()
+        exact = exact and bool(torch.equal(out, want))
+        return {"ms_per_pass": round(ms, 4), "images_per_s": round(xin.shape[0] / (ms * 1e-3), 1),
+                "replays_equal_eager_bitwise": exact}
+    except Exception as e:   # noqa: BLE001
+        try:
+            torch.cuda.synchronize()
+        except Exception:   # noqa: BLE001
+            pass
+        return {"error": "%s: %s" % (type(e).__name__, str(e)[:300])}
 
 
 def main():
@@ -431,7 +487,7 @@ def main():
     ops.set_preexpand(args.preexpand)
 
     if args.network:
-        r = measure_network(pkg, args.network, args.steps, args.warmup, args.fused_layers)
+        r = measure_network(pkg, args.network, args.steps, args.warmup, args.fused_layers, graph=True)
         print(json.dumps({
             "metric": "images_per_s", "value": r["images_per_s"], "unit": "images/s", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "preroll_s": PREROLL_S, "ms_per_step": r["ms_per_pass"],
@@ -439,7 +495,7 @@ def main():
             "config": {"workload": args.network, "input": r["input"], "convolutions": r["convolutions"],
                        "approx_macs_per_pass": r["approx_macs_per_pass"], "fused_layers": r["fused_layers"],
                        "layers_not_fused": r["layers_not_fused"], "note": r["note"]},
-            "approx_gmac_per_s": r["approx_gmac_per_s"]}))
+            "approx_gmac_per_s": r["approx_gmac_per_s"], "hip_graph": r.get("hip_graph")}))
         return
 
     xs, fs, strides, depthwise = WORKLOADS[args.workload]
@@ -603,8 +659,8 @@ def main():
         result["layers_seconds"] = round(time.perf_counter() - t_l, 1)
     if not args.no_networks:
         t_n = time.perf_counter()
-        result["networks"] = [measure_network(pkg, "cifar_resnet_b128", 40, 10),
-                              measure_network(pkg, "resnet50_b64", 12, 3),
+        result["networks"] = [measure_network(pkg, "cifar_resnet_b128", 40, 10, graph=True),
+                              measure_network(pkg, "resnet50_b64", 12, 3, graph=True),
                               measure_network(pkg, "cifar_resnet_b128", 40, 10, fused_layers=True),
                               measure_network(pkg, "resnet50_b64", 12, 3, fused_layers=True)]
         result["networks_seconds"] = round(time.perf_counter() - t_n, 1)
