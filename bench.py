@@ -139,6 +139,7 @@ class Ceilings:
         self.port_bytes = max(ops.lds_read_peak(), 1.0)         # streaming ds_read_b128 bytes/s
         self.valu_lane_ops = max(ops.valu_issue_peak(), 1.0)    # accumulate-instruction lane operations/s
         self.ops_per_lookup = ops.dense_accumulate_ops_per_lookup()
+        self.mix = max(ops.lookup_mix_peak(), 1.0)              # the whole per-lookup instruction mix, lookups/s
         info = ops.device_info()
         self.cus, self.clock_hz = info["compute_units"], info["clock_khz"] * 1e3
         self.valu_nominal = self.cus * 64.0 * self.clock_hz     # 4 SIMDs x 16 lanes per clock and CU
@@ -155,6 +156,7 @@ class Ceilings:
                 "frac_valu": round(f_valu, 4),
                 "frac_lds_port_measured": round(2.0 * lookups_per_s / self.port_bytes, 4),
                 "frac_valu_measured": round(lookups_per_s * self.ops_per_lookup / self.valu_lane_ops, 4),
+                "frac_lookup_mix_measured": round(lookups_per_s / self.mix, 4),
                 "frac_nominal_gather": round(lookups_per_s / NOMINAL_LDS_LOOKUPS_PER_S, 4)}, peak
 
     def report(self):
@@ -166,6 +168,7 @@ class Ceilings:
                 "valu_accumulate_glane_ops_per_s": round(self.valu_lane_ops / 1e9, 1),
                 "valu_ops_per_lookup": self.ops_per_lookup,
                 "valu_glookups_per_s": round(self.valu_lane_ops / self.ops_per_lookup / 1e9, 1),
+                "lookup_mix_glookups_per_s": round(self.mix / 1e9, 1),
                 "valu_nominal_glookups_per_s": round(self.valu_nominal / self.ops_per_lookup / 1e9, 1),
                 "nominal_gather_glookups_per_s": round(NOMINAL_LDS_LOOKUPS_PER_S / 1e9, 1),
                 "measured_ds_read_u16_glookups_per_s": round(self.gather / 1e9, 1),
@@ -579,6 +582,7 @@ def main():
             "frac_valu": fr["frac_valu"],
             "frac_lds_port_measured": fr["frac_lds_port_measured"],
             "frac_valu_measured": fr["frac_valu_measured"],
+            "frac_lookup_mix_measured": fr["frac_lookup_mix_measured"],
             "frac_nominal_gather": fr["frac_nominal_gather"],
             "traffic": traffic,
             "traffic_source": traffic_source,
@@ -588,7 +592,10 @@ def main():
             "note": "frac = the larger of frac_lds_port (2 bytes per lookup against the LDS read port) and frac_valu "
                     "(accumulate instructions per lookup against the vector ALUs' issue rate), each against the larger "
                     "of its nominal ceiling (CUs x 256 B x clock; CUs x 64 lanes x clock) and the rate a probe kernel "
-                    "measured in this run; the *_measured figures are against the probes alone; frac_nominal_gather "
+                    "measured in this run; the *_measured figures are against the probes alone; "
+                    "frac_lookup_mix_measured is against a probe made of the kernel's whole per-lookup instruction mix "
+                    "(address, 16-byte LDS read, accumulate) and nothing else, which neither of the two ceilings "
+                    "contains; frac_nominal_gather "
                     "is against 256 CU x 32 lookups/clk x 2.4 GHz, a ceiling for one-entry gathers that a kernel "
                     "reading 8 entries per access can pass",
             "hbm_algorithmic_bytes": hbm_bytes,

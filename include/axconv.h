@@ -261,6 +261,11 @@ int axc_lds_read_peak(double *bytes_per_second, void *stream);
  * rate / ops_per_lookup is the ceiling the vector ALUs put on lookups per second. */
 int axc_valu_issue_peak(double *lane_ops_per_second, void *stream);
 int axc_dense_accumulate_ops_per_lookup(double *ops);
+/* Rate, in table entries per second over all CUs, of a kernel that contains nothing but the instruction mix of a
+ * LUT-GEMM lookup - address (v_perm_b32), 16-byte LDS read of eight entries, their six accumulate instructions - in
+ * the LUT-GEMM's occupancy.  The LDS read port and the vector ALUs each allow more on their own; a pair of wavefronts
+ * that has to issue both kinds gets this.  No counterpart in the reference (measurement only). */
+int axc_lookup_mix_peak(double *lookups_per_second, void *stream);
 
 /* Properties of the current device the planner uses. */
 int axc_device_info(int *compute_units, int *lds_bytes_per_workgroup, int *clock_khz);

@@ -83,6 +83,7 @@ SYMBOLS = [
     ("axc_lds_gather_peak", ctypes.c_int, [ctypes.POINTER(ctypes.c_double), _vp]),
     ("axc_lds_read_peak", ctypes.c_int, [ctypes.POINTER(ctypes.c_double), _vp]),
     ("axc_valu_issue_peak", ctypes.c_int, [ctypes.POINTER(ctypes.c_double), _vp]),
+    ("axc_lookup_mix_peak", ctypes.c_int, [ctypes.POINTER(ctypes.c_double), _vp]),
     ("axc_dense_accumulate_ops_per_lookup", ctypes.c_int, [ctypes.POINTER(ctypes.c_double)]),
     ("axc_device_info", ctypes.c_int, [ctypes.POINTER(ctypes.c_int)] * 3),
 ]

@@ -1510,6 +1510,15 @@ int axc_valu_issue_peak(double *lane_ops_per_second, void *stream)
     return AXC_OK;
 }
 
+int axc_lookup_mix_peak(double *lookups_per_second, void *stream)
+{
+    if (!lookups_per_second)
+        return fail(AXC_INVALID_ARGUMENT, "null argument");
+    *lookups_per_second = 0.0;
+    AXC_HIP(run_lookup_mix_peak(lookups_per_second, static_cast<hipStream_t>(stream)));
+    return AXC_OK;
+}
+
 int axc_dense_accumulate_ops_per_lookup(double *ops)
 {
     if (!ops)

@@ -245,5 +245,6 @@ hipError_t launch_depthwise_filter(const float *filter, int taps, int C, const T
 hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hipStream_t stream);
 hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128);
 hipError_t run_valu_issue_peak(double *lane_ops_per_second, int mix, hipStream_t stream);
+hipError_t run_lookup_mix_peak(double *lookups_per_second, hipStream_t stream);
 
 } // namespace axc

@@ -462,6 +462,118 @@ hipError_t run_valu_issue_peak(double *lane_ops_per_second, int mix, hipStream_t
     return e;
 }
 
+// The whole instruction mix of a LUT-GEMM lookup instruction, and nothing else: one v_perm_b32 (address), one
+// ds_read_b128 through a rolling window of eight (16 different 16-byte chunks of 256-byte rows per LDS pass: no bank
+// conflict), and the six accumulate instructions of its eight table entries (v_add3_u32 on whole dwords of two
+// lookups, v_add_u32_sdwa on their high halves), in the LUT-GEMM's occupancy (one workgroup of 8 wavefronts and all of
+// the LDS per CU).  Neither the LDS read port nor the vector ALUs alone say what a SIMD can do when a wavefront pair
+// has to issue both kinds: this is the rate a kernel built of exactly these instructions, without fills, activations,
+// barriers, prologue or epilogue, reaches.
+extern __shared__ __align__(16) unsigned char mix_lds[];
+__global__ void __launch_bounds__(kDenseThreads) lookup_mix_probe_kernel(uint32_t *out, int iters)
+{
+    typedef uint32_t u32x4p __attribute__((ext_vector_type(4)));
+    uint32_t *const l32 = reinterpret_cast<uint32_t *>(mix_lds);
+    for (int i = threadIdx.x; i < 32768; i += blockDim.x)
+        l32[i] = (uint32_t)i * 2654435761u;
+    __syncthreads();
+    const uint32_t lane = threadIdx.x & 63u;
+    // a row per lane (any of 256), the lane's own chunk of it: byte 1 of the address comes out of `rows`, byte 0
+    // out of `chunks`, as in the kernels
+    const uint32_t rows = ((lane * 37u) & 255u) * 0x01010101u;
+    const uint32_t chunks = ((lane & 15u) << 4) * 0x01010101u;
+    const uint32_t sel = 0x0c0c0400u;   // byte 0 <- chunks byte 0, byte 1 <- rows byte 0
+    uint32_t acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        acc[i] = threadIdx.x + i;
+    u32x4p v[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        uint32_t a;
+        asm volatile("v_perm_b32 %0, %2, %3, %4\n\tds_read_b128 %1, %0 offset:%5"
+                     : "=&v"(a), "=v"(v[s]) : "v"(rows), "v"(chunks), "v"(sel), "n"(s * 4096));
+    }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int rep = 0; rep < 4; ++rep)
+#pragma unroll
+            for (int s = 0; s < 8; s += 2) {   // two lookup instructions at a time, as the phase bodies do
+                // few, long asm statements: the compiler puts an s_nop between two of them
+                uint32_t *const a = &acc[(s & 2) * 4];
+                const uint32_t x0 = v[s][0], x1 = v[s][1], x2 = v[s][2], x3 = v[s][3];
+                const uint32_t y0 = v[s + 1][0], y1 = v[s + 1][1], y2 = v[s + 1][2], y3 = v[s + 1][3];
+                asm volatile("s_waitcnt lgkmcnt(6)\n\t"
+                             "v_add3_u32 %0, %0, %8, %12\n\t"
+                             "v_add_u32_sdwa %1, %1, %8 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add_u32_sdwa %1, %1, %12 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add3_u32 %2, %2, %9, %13\n\t"
+                             "v_add_u32_sdwa %3, %3, %9 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add_u32_sdwa %3, %3, %13 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add3_u32 %4, %4, %10, %14\n\t"
+                             "v_add_u32_sdwa %5, %5, %10 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add_u32_sdwa %5, %5, %14 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add3_u32 %6, %6, %11, %15\n\t"
+                             "v_add_u32_sdwa %7, %7, %11 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1\n\t"
+                             "v_add_u32_sdwa %7, %7, %15 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_1"
+                             : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7])
+                             : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(y0), "v"(y1), "v"(y2), "v"(y3));
+                uint32_t a0, a1;
+                asm volatile("v_perm_b32 %0, %4, %5, %6\n\tds_read_b128 %2, %0 offset:%7\n\t"
+                             "v_perm_b32 %1, %4, %5, %6\n\tds_read_b128 %3, %1 offset:%8"
+                             : "=&v"(a0), "=&v"(a1), "=&v"(v[s]), "=&v"(v[s + 1])
+                             : "v"(rows), "v"(chunks), "v"(sel), "n"(s * 4096), "n"(s * 4096 + 4096));
+            }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]),
+                 "+v"(v[6]), "+v"(v[7]));
+    uint32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        sum += acc[i];
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        sum += v[s][0] ^ v[s][3];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = sum;
+}
+
+hipError_t run_lookup_mix_peak(double *lookups_per_second, hipStream_t stream)
+{
+    int dev = 0, cus = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    uint32_t *out = nullptr;
+    e = hipMalloc(&out, (size_t)cus * kDenseThreads * sizeof(uint32_t));
+    if (e != hipSuccess) return e;
+    const int lds_bytes = kDenseLdsBytes + kDenseParkBytes;   // what a LUT-GEMM workgroup takes: one workgroup per CU
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(lookup_mix_probe_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    const int iters = 3000;
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(lookup_mix_probe_kernel, dim3(cus), dim3(kDenseThreads), lds_bytes, stream, out, 100);
+        e = hipEventRecord(e0, stream);
+    }
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(lookup_mix_probe_kernel, dim3(cus), dim3(kDenseThreads), lds_bytes, stream, out, iters);
+        e = hipEventRecord(e1, stream);
+    }
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    // 32 lookup instructions per iteration and wavefront, 64 lanes x 8 table entries each
+    if (e == hipSuccess && ms > 0.0f)
+        *lookups_per_second = (double)cus * (kDenseThreads / 64) * (double)iters * 32.0 * 512.0 / (ms * 1e-3);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    return e;
+}
+
 hipError_t run_lds_gather_peak(double *lookups_per_second, hipStream_t stream, bool stream_b128)
 {
     int dev = 0, cus = 0;

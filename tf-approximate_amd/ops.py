@@ -460,6 +460,14 @@ def valu_issue_peak():
     return v.value
 
 
+def lookup_mix_peak():
+    """Table entries per second of a kernel made of nothing but the LUT-GEMM's per-lookup instructions (address,
+    16-byte LDS read, accumulate), in its occupancy (measured)."""
+    v = ctypes.c_double()
+    _check(_lib.load().axc_lookup_mix_peak(ctypes.byref(v), None))
+    return v.value
+
+
 def dense_accumulate_ops_per_lookup():
     v = ctypes.c_double()
     _check(_lib.load().axc_dense_accumulate_ops_per_lookup(ctypes.byref(v)))
