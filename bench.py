@@ -94,8 +94,8 @@ PROFILED_TRAFFIC = {
                                                       "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
     ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 94017.3 * 1024 + 1.000 * 244659.8 * 1024,
                                                       "profiles/lutgemm_px_conv7x7s2_b64_224x224x3_to_64.md"),
-    ("conv3x3_b64_28x28x512_to_512", "lutgemm_expand"): (2.000 * 51701.8 * 1024 + 1.000 * 106354.8 * 1024,
-                                                         "profiles/lutgemm_expand_conv3x3_b64_28x28x512_to_512.md"),
+    ("conv3x3_b64_28x28x512_to_512", "lutgemm_px"): (2.000 * 2065590.0 * 1024 + 1.000 * 106458.5 * 1024,
+                                                     "profiles/lutgemm_px_conv3x3_b64_28x28x512_to_512.md"),
     ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6109.0 * 1024 + 1.025 * 8192.0 * 1024,
                                                     "profiles/lutgemm_px_conv3x3_b128_32x32x16_to_16.md"),
     ("conv1x1_b64_112x112x192_to_32", "lutgemm_px"): (2.000 * 101813.4 * 1024 + 1.000 * 129282.3 * 1024,

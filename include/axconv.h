@@ -150,8 +150,8 @@ int axc_conv2d_tile_plan(const axc_conv2d_desc *desc, int32_t plan[8]);
  * the launch it is for must see the same value. */
 int axc_set_tile_columns(int columns);
 /* Layers with many output pixels per filter element (16-column tiles, an even number of channel quads, whole pairs
- * of fills per K split where K is split, at most 192 MiB of rows) run out of pre-expanded rows: the table rows of every filter element are laid out in the
- * workspace once per call instead of inside every tile.  mode 0 = the planner decides (the default), 1 = every
+ * of fills per K split where K is split, at most 2 GiB of rows) run out of pre-expanded rows: the table rows of
+ * every filter element are laid out in the workspace once per call instead of inside every tile.  mode 0 = the planner decides (the default), 1 = every
  * layer that can run that way does, -1 = none does; process-wide, for tests and timing, initial value from the
  * environment variable AXC_PREEXPAND (read once, when the library is loaded).  Results do not depend on it.  The
  * workspace query counts the rows; a launch whose workspace lacks room for them runs without them, with the tile

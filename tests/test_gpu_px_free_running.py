@@ -7,7 +7,8 @@ the whole tensor of int32 sums and the whole float output bit for bit against th
 (itself pinned against the oracle by the per-layer tests), sampled pixels against the CPU oracle, and, where torch can
 restate the layer, the whole tensor of sums with the exact table against an fp64 convolution of the codes.  Shapes
 cover even and odd fill counts (a tile that starts in LDS buffer 1), a K split, ragged last row tiles, a column count
-that is no multiple of 16, stride, dilation, the flat 7x7x3 layout, both paddings.  The last test forces the kernel's
+that is no multiple of 16, stride, dilation, the flat 7x7x3 layout, both paddings, and a layer whose pre-expanded rows
+(1.2 GB) are larger than any cache.  The last test forces the kernel's
 bounded waits to run out and checks the report."""
 import numpy as np
 import pytest
@@ -33,6 +34,7 @@ CASES = [
     ((32, 56, 56, 64), (3, 3, 64, 20), 1, 1, "SAME"),       # K split in four, 18 fills each
     ((16, 64, 64, 264), (1, 1, 264, 64), 1, 1, "SAME"),     # 1x1, 33 fills (odd)
     ((64, 112, 112, 3), (7, 7, 3, 64), 2, 1, "VALID"),      # flat layout of a 3-channel input, 44-row tiles
+    ((32, 28, 28, 512), (3, 3, 512, 512), 1, 1, "SAME"),    # 1.2 GB of rows: read from memory, not from a cache
 ]
 
 

@@ -168,9 +168,9 @@ def test_tile_plans_fit_the_kernels(ops, lib):
                     assert 1 <= ks <= 16 and (ks - 1) * fps < fills <= ks * fps, what
                 if pl["preexpanded_rows"]:
                     assert mode >= 0 and nt == 16 and fps % 2 == 0 and (xs[3] % 4 or (xs[3] // 4) % 2 == 0), what
-                    assert pl["column_tiles"] * (fps * ks // 2) * 65536 <= (192 << 20) + ks * 65536, what
+                    assert pl["column_tiles"] * (fps * ks // 2) * 65536 <= (2 << 30) + ks * 65536, what
                 elif mode == 1 and nt == 16 and xs[3] % 8 == 0:
-                    assert pl["column_tiles"] * fs[0] * fs[1] * (xs[3] // 8) * 65536 > 192 << 20, what
+                    assert pl["column_tiles"] * fs[0] * fs[1] * (xs[3] // 8) * 65536 > 2 << 30, what
                 if pl["preexpanded_rows"] == 2:
                     # the kernel without barriers keeps its counters in the pixel slot a 64th wavefront-row would
                     # use, and is only picked for tiles of two wavefront-rows per wavefront and 16 fills or more

@@ -433,7 +433,10 @@ std::atomic<int> g_px_mode{[] {
     const int v = env ? std::atoi(env) : 0;
     return (v == 1 || v == -1) ? v : 0;
 }()};
-constexpr size_t kPxMaxBytes = (size_t)192 << 20;   // most memory a layer's pre-expanded rows may take
+constexpr size_t kPxMaxBytes = (size_t)2 << 30;     // most memory a layer's pre-expanded rows may take
+// Rows up to this size stay in the memory-side cache between the launch that writes them and the one that reads
+// them; larger sets are read from memory, and the cost model is less sure of them: they must promise a clear gain.
+constexpr size_t kPxCachedBytes = (size_t)192 << 20;
 
 // Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
 // Derive cost per fill is constant; lookup cost per fill grows with the wavefront-rows a SIMD carries.
@@ -506,8 +509,15 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode, d
                     double px_cost = (double)rounds * ((double)(fps / 2) * (1900.0 + per_simd * 530.0) + 12000.0);
                     if (ks > 1)
                         px_cost = px_cost * 1.08 + split_cost;
+                    double margin = 1.0;
+                    if (px_bytes > (double)kPxCachedBytes) {
+                        // every row comes out of memory at least once (fitted: 3.3 TB/s where no two tiles share rows)
+                        const double stream = px_bytes / 3.3e12 * clock_hz;
+                        px_cost = px_cost > stream ? px_cost : stream;
+                        margin = 0.93;
+                    }
                     px_cost += (6.5e-6 + px_bytes / 5e12) * clock_hz;
-                    if (px_mode > 0 || px_cost < cost) {
+                    if (px_mode > 0 || px_cost < cost * margin) {
                         cost = px_cost;
                         px = 1;
                     }
