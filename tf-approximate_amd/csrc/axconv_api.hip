@@ -774,16 +774,18 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     }
     const bool flat = pd.flat_row_bytes > 0;
     const ConvGeom &gk = pd.gk;   // the layer as the LUT-GEMM kernels and the filter packing see it
-    bool quantized_by_patch_sums = false, filter_done = false;
+    bool quantized_by_patch_sums = false, filter_done = false, px_done = false;
+    uint16_t *const px_rows = use_px ? reinterpret_cast<uint16_t *>(ws + pd.ws.px_off) : nullptr;
     if (out_f && !codes_mode) {
-        ProfScope ps(flat ? "patch_sums_flat" : "patch_sums", stream);   // carries the filter pre-pass along when it can
-        const FilterJob job = {filter, filter_codes, &pd.plan, tq_f, wq, fsum};
+        // carries the filter pre-pass, and with it the pre-expanded rows, along when it can
+        ProfScope ps(flat ? "patch_sums_flat" : "patch_sums", stream);
+        const FilterJob job = {filter, filter_codes, &pd.plan, tq_f, wq, fsum, table->dev_tableT, px_rows};
         if (flat)   // the patch sums write the flat layout where they hold the rows anyway, else the pass below does
             AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, nullptr,
                                       nullptr, pd.flat_row_bytes));
         else
             AXC_HIP(launch_patch_sums(input, g, tq_in, lq_dev, psum, stream, xq, &quantized_by_patch_sums, &job,
-                                      &filter_done));
+                                      &filter_done, 0, &px_done));
     }
     if (flat && !quantized_by_patch_sums) {
         ProfScope ps("quantize_flat_rows", stream);
@@ -838,10 +840,11 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     p.spin_limit = g_wait_limit.load(std::memory_order_relaxed);
     p.wait_error = wait_word;
     if (use_px) {
-        ProfScope ps("px_expand_rows", stream);
-        uint16_t *rows = reinterpret_cast<uint16_t *>(ws + pd.ws.px_off);
-        AXC_HIP(launch_px_expand_rows(wq, table->dev_tableT, pd.plan, rows, stream));
-        p.px_rows = rows;
+        if (!px_done) {
+            ProfScope ps("px_expand_rows", stream);
+            AXC_HIP(launch_px_expand_rows(wq, table->dev_tableT, pd.plan, px_rows, stream));
+        }
+        p.px_rows = px_rows;
         p.px_bytes = (uint32_t)pd.ws.px_bytes;
     }
     if (flat) {

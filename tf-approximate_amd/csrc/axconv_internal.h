@@ -204,13 +204,17 @@ struct FilterJob {
     TensorQuant tq;
     uint16_t *wq;
     float *fsum;
+    const uint16_t *tableT;   // with px_rows: the transposed table the pre-expanded rows are built from
+    uint16_t *px_rows;        // nullptr: the layer does not run out of pre-expanded rows
 };
 // xq_fused / fused: the launch may also quantize the input into xq (then *fused is set);
-// filter_job / filter_done: it may also do the filter pre-pass (then *filter_done is set).
+// filter_job / filter_done: it may also do the filter pre-pass (then *filter_done is set), and with it build the
+// pre-expanded rows that filter_job names (then *px_done is set).
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
                              float *psum, hipStream_t stream, uint32_t *xq_fused = nullptr, bool *fused = nullptr,
                              const FilterJob *filter_job = nullptr, bool *filter_done = nullptr,
-                             int flat_row_bytes = 0);   // > 0: a fused xq is written in the flat layout
+                             int flat_row_bytes = 0,   // > 0: a fused xq is written in the flat layout
+                             bool *px_done = nullptr);
 hipError_t launch_layer_quant(const float *input, int64_t n_input, const float *filter, int64_t n_filter, int K,
                               float *partials, LayerQuant *lq_dev, hipStream_t stream);
 constexpr int kMinMaxBlocks = 2048;   // partial (min, max) pairs per tensor in launch_layer_quant's scratch

@@ -19,52 +19,30 @@
 // Restates ApproxConvIm2ColKernel + ApproxConvGEMMKernel (tf2/src/approx_nn_conv_kernels.cpp:215-296) like the
 // other kernel; results are bit-identical to it (same int32 sums, same epilogue).
 #include "lutgemm_tile.h"
+#include "px_expand.h"
 #include "lookup_asm.inc"
 
 namespace axc {
 
 extern __shared__ __align__(16) unsigned char lds_px[];
 
-constexpr int kPxFillBytes = 65536;     // one pre-expanded fill: 256 activation rows x 128 slots x uint16
 constexpr int kPxBlockCols = 4;         // column tiles that the workgroups of an XCD walk side by side
 
-// One workgroup per (column tile, fill, part): a part is 256 / kPxExpandParts activation codes, four threads each.
-// Thread (a, quarter) gathers 32 of the 128 entries of activation code a - 32 independent two-byte loads out of the
-// L2-resident table, coalesced over a - into LDS (row a, 65 dwords apart: no bank conflicts); then every wavefront
-// copies whole 256-byte rows to memory, one row per store instruction, to the rows phys_row() gives the codes.
-// Parts rather than whole fills: several workgroups fit a CU, so a layer's few hundred fills spread evenly over the
-// CUs instead of as one round and a remainder.
-constexpr int kPxExpandPitch = 65;   // dwords per activation row in LDS
+// One workgroup per (column tile, fill, part): see px_expand.h.
 constexpr int kPxExpandParts = 2;
 constexpr int kPxExpandCodes = 256 / kPxExpandParts;
 __global__ void __launch_bounds__(4 * kPxExpandCodes) px_expand_rows_kernel(const uint16_t *__restrict__ wq,
                                                                             const uint16_t *__restrict__ tableT,
                                                                             const int fills, uint16_t *__restrict__ rows)
 {
-    __shared__ uint32_t stage[kPxExpandCodes * kPxExpandPitch];
+    __shared__ uint32_t stage[px_expand_stage_dwords<kPxExpandCodes>()];
     const int px_fills = fills / 2;
     const int part = (int)blockIdx.x % kPxExpandParts, cf = (int)blockIdx.x / kPxExpandParts;   // cf = ct * px_fills + f
     const int ct = cf / px_fills, f = cf - ct * px_fills;
-    const uint32_t al = threadIdx.x % kPxExpandCodes, a = (uint32_t)part * kPxExpandCodes + al;
-    const int quarter = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kPxExpandCodes));
     // the codes of the two ordinary fills of this pair lie side by side: 128 uint16
-    const uint16_t *codes = wq + ((size_t)ct * fills + 2 * (size_t)f) * 64 + quarter * 32;
-#pragma unroll
-    for (int d = 0; d < 16; ++d) {
-        const uint32_t lo = tableT[(uint32_t)codes[2 * d] * 256u + a];
-        const uint32_t hi = tableT[(uint32_t)codes[2 * d + 1] * 256u + a];
-        stage[al * kPxExpandPitch + quarter * 16 + d] = lo | (hi << 16);
-    }
-    __syncthreads();
-    uint32_t *const dst = reinterpret_cast<uint32_t *>(rows + (size_t)cf * (kPxFillBytes / 2));
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    constexpr int kWaves = 4 * kPxExpandCodes / 64, kPer = kPxExpandCodes / kWaves;
-#pragma unroll
-    for (int i = 0; i < kPer; ++i) {
-        const uint32_t cl = wave * kPer + i;                     // code of this part
-        const uint32_t code = (uint32_t)part * kPxExpandCodes + cl;
-        dst[phys_row(code) * 64u + lane] = stage[cl * kPxExpandPitch + lane];
-    }
+    const uint16_t *codes = wq + ((size_t)ct * fills + 2 * (size_t)f) * 64;
+    px_expand_part<kPxExpandCodes>(stage, part, [&](const int s) { return codes[s]; }, tableT,
+                                   reinterpret_cast<uint32_t *>(rows + (size_t)cf * (kPxFillBytes / 2)));
 }
 
 hipError_t launch_px_expand_rows(const uint16_t *wq, const uint16_t *tableT, const DensePlan &plan, uint16_t *rows,

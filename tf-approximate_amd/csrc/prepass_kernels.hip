@@ -1,5 +1,7 @@
 // Pre-pass kernels: quantize + relayout of the input, filter quantize/pack/sums, flat quantize.
 #include "axconv_internal.h"
+#include "px_expand.h"
+#include <type_traits>
 
 namespace axc {
 
@@ -248,6 +250,12 @@ struct FilterWork {
     // pack_total > 0: no pack blocks; the threads of the patch-sum blocks that run no chain pack the codes,
     // each block its share of the pack_total elements
     int64_t pack_total;
+    // expand_blocks > 0: the last workgroups of the launch build the pre-expanded rows of lutgemm_px_kernel.hip
+    // (px_expand.h), blockDim.x / 4 activation codes of one (column tile, pair of fills) each: the rows depend on the
+    // filter and the table only, so they need not wait for the patch sums in a launch of their own
+    int expand_blocks;
+    const uint16_t *tableT;
+    uint16_t *px_rows;
 };
 
 __device__ __forceinline__ void filter_pack_element(const int64_t i, const float *__restrict__ filter,
@@ -637,16 +645,14 @@ __global__ void __launch_bounds__(256) codes_relayout_kernel(const uint8_t *__re
 // and pack into the order the LUT-GEMM consumes.
 //   wq[ct][fill][slot], fill = (tap * C4 + q) * SUBS + sub, slot = kk * NT + j
 //   channel = q*4 + sub*KS + kk, column = ct*NT + j; kNullWeight where channel >= C or column >= Co.
-__device__ __forceinline__ void filter_pack_element(const int64_t i, const float *__restrict__ filter,
-                                                    const uint8_t *__restrict__ filter_codes, int taps, int C,
-                                                    int C4, int Co, int nt, int n_col_tiles, const TensorQuant &qf,
-                                                    uint16_t *__restrict__ wq)
+// Element i of the packed filter [column tile][fill][slot]: the code of the filter element the slot stands for, the
+// null weight where the slot is padding (i < column tiles x fills x 64).
+__device__ __forceinline__ uint16_t filter_code_at(const int64_t i, const float *__restrict__ filter,
+                                                   const uint8_t *__restrict__ filter_codes, int taps, int C, int C4,
+                                                   int Co, int nt, const TensorQuant &qf)
 {
     const int ks = 64 / nt, subs = 4 / ks;
     const int fills = taps * C4 * subs;
-    const int64_t total = (int64_t)n_col_tiles * fills * 64;
-    if (i >= total)
-        return;
     const int slot = (int)(i & 63);
     const int64_t f = i >> 6;
     const int fill = (int)(f % fills);
@@ -664,7 +670,17 @@ __device__ __forceinline__ void filter_pack_element(const int64_t i, const float
         code = filter_codes ? (uint16_t)filter_codes[idx]
                             : (uint16_t)quantize_code(fake_quant_value(filter[idx], qf), qf.offset, qf.inv_scale);
     }
-    wq[i] = code;
+    return code;
+}
+
+__device__ __forceinline__ void filter_pack_element(const int64_t i, const float *__restrict__ filter,
+                                                    const uint8_t *__restrict__ filter_codes, int taps, int C,
+                                                    int C4, int Co, int nt, int n_col_tiles, const TensorQuant &qf,
+                                                    uint16_t *__restrict__ wq)
+{
+    const int64_t total = (int64_t)n_col_tiles * (taps * C4 * (nt / 16)) * 64;
+    if (i < total)
+        wq[i] = filter_code_at(i, filter, filter_codes, taps, C, C4, Co, nt, qf);
 }
 
 // Filter sums (tf2/src/approx_nn_conv_kernels.cpp:300-306): one sequential sum per output column, rows (h, w, c)
@@ -1040,8 +1056,35 @@ __device__ __forceinline__ bool filter_work_block(const FilterWork &fw, const La
     if (*bid < fw.work_blocks)
         return false;
     const TensorQuant q = lq_dev ? lq_dev->flt : fw.tq;
-    const int64_t i = (int64_t)(*bid - fw.work_blocks) * blockDim.x + threadIdx.x;
-    filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+    const int pb = *bid - fw.work_blocks;
+    if (pb < fw.pack_blocks || fw.expand_blocks == 0) {
+        const int64_t i = (int64_t)pb * blockDim.x + threadIdx.x;
+        filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
+        return true;
+    }
+    // pre-expanded rows (16-column tiles: a fill is one channel quad of a tap, fills = taps x C4): this workgroup
+    // computes the 128 filter codes of its pair of fills into LDS, then expands them
+    extern __shared__ __align__(16) unsigned char px_lds[];
+    const int eb = pb - fw.pack_blocks;
+    const int fills = fw.taps * fw.C4, px_fills = fills / 2;
+    uint32_t *const stage = reinterpret_cast<uint32_t *>(px_lds);
+    const auto body = [&](auto cb_tag) {
+        constexpr int CB = decltype(cb_tag)::value;
+        constexpr int kParts = 256 / CB;
+        const int part = eb % kParts, cf = eb / kParts;   // cf = ct * px_fills + f
+        const int ct = cf / px_fills, f = cf - ct * px_fills;
+        uint16_t *const codes = reinterpret_cast<uint16_t *>(stage + px_expand_stage_dwords<CB>());
+        if (threadIdx.x < 128)
+            codes[threadIdx.x] = filter_code_at(((int64_t)ct * fills + 2 * (int64_t)f) * 64 + threadIdx.x, fw.filter,
+                                                fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, 16, q);
+        __syncthreads();
+        px_expand_part<CB>(stage, part, [&](const int sl) { return codes[sl]; }, fw.tableT,
+                           reinterpret_cast<uint32_t *>(fw.px_rows + (size_t)cf * (kPxFillBytes / 2)));
+    };
+    if (blockDim.x == 512)
+        body(std::integral_constant<int, 128>());
+    else
+        body(std::integral_constant<int, 256>());
     return true;
 }
 
@@ -1552,12 +1595,14 @@ static void choose_band(const ConvGeom &g, int sum_blocks, int *rb_out, int *in_
 
 hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuant &tq, const LayerQuant *lq_dev,
                              float *psum, hipStream_t stream, uint32_t *xq_fused, bool *fused,
-                             const FilterJob *filter_job, bool *filter_done, int flat_row_bytes)
+                             const FilterJob *filter_job, bool *filter_done, int flat_row_bytes, bool *px_done)
 {
     if (fused)
         *fused = false;
     if (filter_done)
         *filter_done = false;
+    if (px_done)
+        *px_done = false;
     const bool vec = (g.C & 3) == 0 && ((uintptr_t)x & 15) == 0;
     if (flat_row_bytes && vec)   // the flat layout belongs to channel counts that are no multiple of four
         return hipErrorInvalidValue;
@@ -1647,9 +1692,31 @@ hipError_t launch_patch_sums(const float *x, const ConvGeom &g, const TensorQuan
                 if (fw.sum_blocks && lds < (size_t)kFsLdsBytes)
                     lds = kFsLdsBytes;
                 *filter_done = true;
+                // ... and so do the pre-expanded rows where the layer runs out of them: blockDim.x / 4 activation
+                // codes of a pair of fills per workgroup, the stage and the pair's 128 filter codes in LDS
+                if (px_done && filter_job->px_rows && plan.nt == 16 && plan.fills == fw.taps * fw.C4 &&
+                    (plan.fills & 1) == 0) {
+                    const int64_t eb = (int64_t)plan.n_col_tiles * (plan.fills / 2) * (1024 / block_threads);
+                    const size_t need = (size_t)(block_threads / 4) * kPxExpandPitch * 4 + 256;
+                    // Every workgroup of a launch takes the same LDS.  Where the patch sums take so much that a CU
+                    // holds fewer of these workgroups than its wavefront slots allow (2048 threads), the rows are
+                    // written more slowly; that still beats a launch of their own (north star -1.8 %, 3x3 128->128
+                    // @28x28 -3.1 %) until the rows are many (1.2 GB: 0.26 -> 0.33 ms, +2.3 % on the layer).
+                    const size_t lds_with = lds < need ? need : lds;
+                    const bool slow = lds_with * (size_t)(2048 / block_threads) > (size_t)device_lds_bytes();
+                    const size_t row_bytes = (size_t)plan.n_col_tiles * (size_t)(plan.fills / 2) * kPxFillBytes;
+                    if (eb + fw.sum8 + work_blocks + fw.pack_blocks < ((int64_t)1 << 31) &&
+                        lds_with <= (size_t)device_lds_bytes() && !(slow && row_bytes > ((size_t)512 << 20))) {
+                        fw.expand_blocks = (int)eb;
+                        fw.tableT = filter_job->tableT;
+                        fw.px_rows = filter_job->px_rows;
+                        lds = lds < need ? need : lds;
+                        *px_done = true;
+                    }
+                }
             }
             fw.work_blocks = (int)work_blocks;
-            const unsigned grid = (unsigned)(fw.sum8 + work_blocks + fw.pack_blocks);
+            const unsigned grid = (unsigned)(fw.sum8 + work_blocks + fw.pack_blocks + fw.expand_blocks);
             if (segmented) {
                 const hipError_t e =
                     set_max_dynamic_lds_once(reinterpret_cast<const void *>(patch_sums_segments_kernel), device_lds_bytes());
