@@ -435,7 +435,7 @@ std::atomic<int> g_px_mode{[] {
 }()};
 constexpr size_t kPxMaxBytes = (size_t)2 << 30;     // most memory a layer's pre-expanded rows may take
 // Rows up to this size stay in the memory-side cache between the launch that writes them and the one that reads
-// them; larger sets are read from memory, and the cost model is less sure of them: they must promise a clear gain.
+// them; larger sets are read from memory, and the cost model is less sure of them: they must promise a gain.
 constexpr size_t kPxCachedBytes = (size_t)192 << 20;
 
 // Tile plan: columns per tile (16/32/64) and rows per tile, by a cost model in LDS/VALU cycles.
@@ -480,8 +480,11 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode, d
         for (int64_t n_row : cands) {
             const int64_t wrows = (total_wrows + n_row - 1) / n_row;  // per tile
             const double per_simd = (double)((wrows + 3) / 4);          // wavefront-rows on the busiest SIMD
-            // cycles per fill, fitted to measurements: barrier + expanding + staging, then the lookups
-            const double per_fill = 1700.0 + per_simd * 290.0;
+            // Cycles, fitted to the LUT-GEMM launch times of ~85 layer shapes run both ways (mean error 3.5 %).
+            // Per fill: barrier + expanding + staging, then the lookups; per tile: geometry, the first fills, the
+            // turn and store of the outputs, which grow with the tile's rows.  (What a launch costs whatever its
+            // plan, ~25 000 cycles, is left out.)
+            const double per_fill = 1658.0 + per_simd * 247.0;
             // Splitting K over tiles keeps the tiles tall (many lookups per expanded fill) when M alone does not
             // give every CU a tile; the int32 partial sums then cost one more pass over (k_splits + 1) outputs.
             for (int ks : {1, 2, 3, 4, 6, 8, 12, 16}) {
@@ -494,29 +497,25 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode, d
                     continue;
                 const int64_t tiles = n_row * n_col * ks;
                 const int64_t rounds = (tiles + cus - 1) / cus;
-                double cost = (double)rounds * ((double)fps * per_fill + 6000.0);
-                // the extra pass of a K split, and a margin: split only for a clear gain
-                const double split_cost = ks > 1 ? 20000.0 + (double)(ks + 1) * (double)g.M * g.Co * 4.0 * 7e-4 : 0.0;
-                if (ks > 1)
-                    cost = cost * 1.08 + split_cost;
+                double cost = (double)rounds * ((double)fps * per_fill + 2200.0 + per_simd * 1876.0);
+                // the extra pass of a K split (fitted: 13 900 cycles + 6.8 TB/s), and a margin: split only for a gain
+                const double split_cost = ks > 1 ? 17000.0 + (double)(ks + 1) * (double)g.M * g.Co * 4.0 * 3.5e-4 : 0.0;
+                cost += split_cost;
                 // The same tiles out of pre-expanded rows (16 columns, whole K, channel quads in pairs): a phase
-                // covers two fills and neither expands nor stages (fitted: 8 300 cycles at 13 wavefront-rows per
-                // SIMD, 2 900 at 2); the rows cost 512 bytes of memory per filter element, written once per call by
-                // one more launch (~6.5 us, then ~5 TB/s).
+                // covers two fills and neither expands nor stages (8 200 cycles at 13 wavefront-rows per SIMD,
+                // 2 800 at 2).  The rows cost 512 bytes of memory per filter element, written once per call: by
+                // workgroups that ride in the patch-sum launch (measured: +1.5 us, then 7 TB/s), beyond ~400 MB
+                // more slowly or by a launch of their own (6.5 us, 4.5 TB/s); and every row comes out of memory at
+                // least once, at 3 TB/s where no two tiles share rows.  Sets too large to stay in the memory-side
+                // cache between the two launches must promise 2 %.
                 int px = 0;
                 if (px_possible && px_mode >= 0 && nt == 16 && (ks == 1 || (fps & 1) == 0)) {
                     const double px_bytes = (double)n_col * (double)(fills / 2) * 65536.0;
-                    double px_cost = (double)rounds * ((double)(fps / 2) * (1900.0 + per_simd * 530.0) + 12000.0);
-                    if (ks > 1)
-                        px_cost = px_cost * 1.08 + split_cost;
-                    double margin = 1.0;
-                    if (px_bytes > (double)kPxCachedBytes) {
-                        // every row comes out of memory at least once (fitted: 3.3 TB/s where no two tiles share rows)
-                        const double stream = px_bytes / 3.3e12 * clock_hz;
-                        px_cost = px_cost > stream ? px_cost : stream;
-                        margin = 0.93;
-                    }
-                    px_cost += (6.5e-6 + px_bytes / 5e12) * clock_hz;
+                    double px_cost = (double)rounds * ((double)(fps / 2) * (1790.0 + per_simd * 493.0) + per_simd * 1980.0);
+                    const double stream = px_bytes / 3.0e12 * clock_hz;
+                    px_cost = (px_cost > stream ? px_cost : stream) + split_cost;
+                    const double margin = px_bytes > (double)kPxCachedBytes ? 0.98 : 1.0;
+                    px_cost += (px_bytes <= 400e6 ? 1.5e-6 + px_bytes / 7e12 : 6.5e-6 + px_bytes / 4.5e12) * clock_hz;
                     if (px_mode > 0 || px_cost < cost * margin) {
                         cost = px_cost;
                         px = 1;
