@@ -220,6 +220,8 @@ def test_rows_are_built_by_the_pre_pass_launch_where_it_can_carry_them(pkg, orac
         for xs, fs, strides, own_launch in (((3, 20, 20, 16), (3, 3, 16, 24), (1, 1), False),
                                             ((2, 30, 30, 64), (1, 1, 64, 40), (1, 1), False),     # flat pixel list
                                             ((2, 14, 14, 512), (1, 1, 512, 16), (1, 1), False),   # few pixels, many channels
+                                            ((4, 300, 300, 8), (3, 3, 8, 16), (1, 1), False),     # bands of 900 pixels: workgroups
+                                                                                                    # of 1024, a whole fill each
                                             ((2, 40, 40, 3), (7, 7, 3, 16), (2, 2), True)):
             x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=sum(xs))
             op = pkg.ApproxConv2DWithMinMaxVars([1, strides[0], strides[1], 1], 8, table, "SAME")
