@@ -88,9 +88,9 @@ PROFILED_TRAFFIC = {
                                                                "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
     ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48253.9 * 1024 + 1.000 * 790871.3 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b64_112x112x32_to_192.md"),
-    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37230.7 * 1024 + 1.000 * 267278.5 * 1024,
+    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37308.6 * 1024 + 1.000 * 267897.6 * 1024,
                                                     "profiles/lutgemm_px_conv1x1_b64_56x56x64_to_256.md"),
-    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 470745.2 * 1024 + 1.000 * 471721.4 * 1024,
+    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 471479.0 * 1024 + 1.000 * 470258.6 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
     ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 94017.6 * 1024 + 1.000 * 245457.2 * 1024,
                                                       "profiles/lutgemm_px_conv7x7s2_b64_224x224x3_to_64.md"),
@@ -98,7 +98,7 @@ PROFILED_TRAFFIC = {
                                                      "profiles/lutgemm_px_conv3x3_b64_28x28x512_to_512.md"),
     ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6109.0 * 1024 + 1.025 * 8192.0 * 1024,
                                                     "profiles/lutgemm_px_conv3x3_b128_32x32x16_to_16.md"),
-    ("conv1x1_b64_112x112x192_to_32", "lutgemm_px"): (2.000 * 101813.3 * 1024 + 1.000 * 129824.0 * 1024,
+    ("conv1x1_b64_112x112x192_to_32", "lutgemm_px"): (2.000 * 101813.4 * 1024 + 1.000 * 129997.3 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b64_112x112x192_to_32.md"),
     ("conv3x3_b64_28x28x128_to_128", "lutgemm_px"): (2.000 * 130201.6 * 1024 + 1.000 * 54427.9 * 1024,
                                                      "profiles/lutgemm_px_conv3x3_b64_28x28x128_to_128.md"),

@@ -838,16 +838,20 @@ __device__ __forceinline__ void patch_sums_flat_body(const float *__restrict__ x
     constexpr int QUADS = kFlatChunk / 4, PSTEP = kFlatThreads / QUADS;
     const int q = t % QUADS, px0 = t / QUADS;
     const bool copier = t < kFlatThreads;
-    uint32_t xq_idx[kFlatPer];        // dword index in xq of (pixel, quad q of chunk 0)
-    int64_t x_idx[kFlatPer];          // float index in x of the same
+    int64_t x_idx[kFlatPer];          // float index in x of (pixel, quad q of chunk 0)
 #pragma unroll
     for (int k = 0; k < kFlatPer; ++k) {
         const int px = px0 + k * PSTEP;    // k beyond pixels / PSTEP: px >= npx, nothing loaded or stored
         const int64_t m = m0 + (px < npx ? px : 0);
-        const int64_t nh = m / g.W;
-        const int w = (int)(m - nh * g.W);
-        xq_idx[k] = (uint32_t)((nh * g.C4 + q) * g.W + w);
         x_idx[k] = m * g.C + q * 4;
+    }
+    // ... and thread -> (pixel, first quad) for the codes: pixel t % pixels, quads t / pixels, + kFlatThreads / pixels, ...
+    const int code_px = t % pixels, code_q0 = t / pixels, code_qstep = kFlatThreads / pixels;
+    uint32_t code_idx = 0;            // dword index in xq of (that pixel, quad 0)
+    {
+        const int64_t m = m0 + (code_px < npx ? code_px : 0);
+        const int64_t nh = m / g.W;
+        code_idx = (uint32_t)(nh * g.C4 * g.W + (m - nh * g.W));
     }
     const int chunks = (g.C + kFlatChunk - 1) / kFlatChunk;
     float4 v[kFlatPer];
@@ -870,19 +874,26 @@ __device__ __forceinline__ void patch_sums_flat_body(const float *__restrict__ x
                 const int px = px0 + k * PSTEP;
                 if (px >= pixels)
                     continue;
-                const float4 f = fake_quant_value4(v[k], qt);
-                *reinterpret_cast<float4 *>(&rows[px * kFlatPitch + q * 4]) = f;
-                if (xq && px < npx && c0 + q * 4 < g.C)
-                    xq[xq_idx[k] + (uint32_t)(c0 / 4) * (uint32_t)g.W] =
-                        phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
-                        (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
-                        (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
-                        (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
+                *reinterpret_cast<float4 *>(&rows[px * kFlatPitch + q * 4]) = fake_quant_value4(v[k], qt);
             }
         }
         __syncthreads();
         if (ch + 1 < chunks)
             load_chunk(c0 + kFlatChunk);
+        if (xq && copier && code_px < npx) {
+            // The codes go out of LDS, not out of the registers the floats came in: there a wavefront holds 16 quads
+            // of 4 pixels, and a quad's codes lie a row of W dwords apart in xq - 16 runs of 16 bytes per store;
+            // here it holds one quad of 64 consecutive pixels: one run of 256 bytes.
+            const int nq = (g.C - c0 < kFlatChunk ? g.C - c0 : kFlatChunk) / 4;
+            for (int qq = code_q0; qq < nq; qq += code_qstep) {
+                const float4 f = *reinterpret_cast<const float4 *>(&rows[code_px * kFlatPitch + qq * 4]);
+                xq[code_idx + (uint32_t)(c0 / 4 + qq) * (uint32_t)g.W] =
+                    phys_row(quantize_code(f.x, qt.offset, qt.inv_scale)) |
+                    (phys_row(quantize_code(f.y, qt.offset, qt.inv_scale)) << 8) |
+                    (phys_row(quantize_code(f.z, qt.offset, qt.inv_scale)) << 16) |
+                    (phys_row(quantize_code(f.w, qt.offset, qt.inv_scale)) << 24);
+            }
+        }
         if (t < npx) {
             const int nq = (g.C - c0 < kFlatChunk ? g.C - c0 : kFlatChunk) / 4;
             const float *src = &rows[t * kFlatPitch];
