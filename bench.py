@@ -388,8 +388,8 @@ def measure_network(pkg, name, steps, warmup, fused_layers=False, graph=False):
            "ms_per_pass": round(ms, 4), "images_per_s": round(xin.shape[0] / (ms * 1e-3), 1),
            "approx_macs_per_pass": macs, "approx_gmac_per_s": round(macs / (ms * 1e-3) / 1e9, 1),
            "fused_layers": bool(fused_layers), "layers_not_fused": net.unfused_layers() if fused_layers else [],
-           "note": "convolutions through the op, a ReLU that directly follows one fused into its store; adds (with their ReLU) "
-                   "and the max-pool in torch"}
+           "note": "convolutions through the op, a ReLU that directly follows one fused into its store; each add with its "
+                   "ReLU as one torch elementwise kernel (torch.cuda.jiterator) and the max-pool in torch"}
     if graph:
         rec["hip_graph"] = graph_replay(net, xin, steps)
     return rec

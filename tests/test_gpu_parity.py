@@ -319,6 +319,19 @@ def test_network_layers_vs_oracle(pkg, oracle, name):
         assert refimpl.linf_rel(y, y_ref) <= 1e-5
 
 
+def test_harness_add_relu_is_torchs(pkg):
+    """The network harness adds a shortcut and applies the ReLU in one elementwise kernel: same bits as torch's two."""
+    import torch
+    from tf_approximate_amd import networks
+    g = torch.Generator(device=gpu_util.dev()).manual_seed(3)
+    a = torch.randn((3, 17, 19, 24), generator=g, device=gpu_util.dev())
+    b = torch.randn((3, 17, 19, 24), generator=g, device=gpu_util.dev())
+    a[0, 0, 0, :4] = torch.tensor([float("nan"), float("inf"), -float("inf"), -0.0], device=gpu_util.dev())
+    want = torch.relu(a + b)
+    got = networks.add_relu(a.clone(), b)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+
+
 def test_split_k_plan_is_exercised(pkg):
     """The cases above named for it really run with K split over tiles (and the north-star layer does not)."""
     from tf_approximate_amd import ops

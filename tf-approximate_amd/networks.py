@@ -10,7 +10,8 @@ forward pass from layer lists, random He-normal weights and synthetic inputs:
     inverted_residual  MobileNetV2-style block: 1x1 expand (x6), depthwise 3x3 (stride 1 or 2), 1x1 project
 
 Only the convolutions run through the library (with the ReLU that directly follows one fused into its store);
-residual adds with their ReLU and the max-pool are torch glue.  The
+residual adds with their ReLU (one elementwise kernel built by torch.cuda.jiterator, or torch's add and relu where
+that is not available) and the max-pool are torch glue.  The
 min/max of every layer input and filter are taken from the tensors in a calibration pass (the Keras wrapper's
 policy) and then held fixed, so the timed pass has no host synchronisation.
 """
@@ -20,6 +21,26 @@ import numpy as np
 import torch
 
 from . import ops
+
+
+_ADD_RELU = None
+
+
+def add_relu(a, b):
+    """relu(a + b) as one elementwise kernel: torch compiles the functor at its first use (hiprtc) and caches it.
+    Same values as torch.relu(a + b), NaNs included; falls back to torch's two kernels where the JIT is unavailable."""
+    global _ADD_RELU
+    if _ADD_RELU is None:
+        try:
+            fn = torch.cuda.jiterator._create_jit_fn(
+                "template <typename T> T add_relu(T a, T b) { T s = a + b; return s > T(0) ? s : (s == s ? T(0) : s); }")
+            fn(a, b)
+            _ADD_RELU = fn
+        except Exception:   # no JIT on this build: torch's own kernels
+            _ADD_RELU = False
+    if _ADD_RELU is False:
+        return torch.relu_(a.add_(b))
+    return _ADD_RELU(a, b)
 
 
 class ConvSpec:
@@ -107,8 +128,8 @@ class ApproxNetwork:
                     y = self.ops[i](src, w, *self.ranges[i], activation="relu" if spec.relu else None)
                 macs += spec.macs(y.shape[1], y.shape[2], y.shape[0])
                 t[dst] = y
-            elif kind == "add_relu":   # the first operand is a convolution's fresh output: added to in place
-                t[dst] = torch.relu_(t[step[2]].add_(t[step[3]]))
+            elif kind == "add_relu":
+                t[dst] = add_relu(t[step[2]], t[step[3]])
             elif kind == "maxpool":
                 nchw = t[step[2]].permute(0, 3, 1, 2)
                 t[dst] = torch.nn.functional.max_pool2d(nchw, 3, 2, 1).permute(0, 2, 3, 1).contiguous()
