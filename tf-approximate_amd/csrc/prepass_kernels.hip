@@ -421,12 +421,12 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
     const int iw0 = ow * g.sw - g.pw;
     float s = 0.0f;
     __builtin_amdgcn_s_setprio(3);   // the chain is the critical path: its wavefront issues ahead of the others on its SIMD
-    if ((g.C4 & 7) == 0) {
+    const auto batched_chain = [&](auto batch_tag) {
         // The chain of K dependent adds is what takes the time here, so nothing else may wait on it: the taps and
-        // their channels form one flat list of batches of 32 floats, the LDS reads of a batch are issued a batch
+        // their channels form one flat list of batches of 32 floats (16 where the channel quads are no multiple of 8), the LDS reads of a batch are issued a batch
         // ahead of its adds, and every lane takes every tap - a tap outside the image reads the pixel of zeros
         // (x + 0 == x; the sum starts at +0 and so is never -0) instead of branching around it.
-        constexpr int kBatch = 8; // 16-byte reads per batch
+        constexpr int kBatch = decltype(batch_tag)::value; // 16-byte reads per batch: 8, or 4 for 16 channels and the like
         const int bpt = g.C4 / kBatch, nb = g.KH * g.KW * bpt;
         int kh = 0, kw = 0, bi = 0;
         auto tap_src = [&]() -> const float4 * {
@@ -475,6 +475,13 @@ __device__ __forceinline__ void patch_sums_rows_body(const float *__restrict__ x
             chain_fence(s);
         }
         psum[((int64_t)n * g.OH + oh) * g.OW + ow] = s;
+    };
+    if ((g.C4 & 7) == 0) {
+        batched_chain(std::integral_constant<int, 8>());
+        return;
+    }
+    if ((g.C4 & 3) == 0) {
+        batched_chain(std::integral_constant<int, 4>());
         return;
     }
     for (int kh = 0; kh < g.KH; ++kh) {
