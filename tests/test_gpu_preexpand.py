@@ -206,23 +206,25 @@ def test_planner_picks_preexpanded_rows_for_many_pixels_only(pkg):
         ops.profile_enable(False)
 
 
-def test_rows_are_built_by_the_pre_pass_launch_where_it_can_carry_them(pkg, oracle):
-    """Float inputs with a channel count that is a multiple of four: the patch-sum launch also quantizes the input,
-    packs the filter and builds the pre-expanded rows, so the library's kernel timers show no launch of
-    px_expand_rows_kernel.  Integer-code inputs (no patch sums) and the flat 3-channel layout (patch sums by a kernel
-    that carries no filter work) still get that launch.  All three are checked against the oracle, so rows built
-    either way are the same rows."""
+def test_rows_are_built_by_the_pre_pass_launches(pkg, oracle):
+    """The pre-expanded rows depend on the filter and the table only, so they are built by further workgroups of a
+    launch that is there anyway: the patch-sum launch (float inputs with a multiple of four channels: bands, flat
+    pixel list, few pixels of many channels, workgroups of 512 and of 1024), else the filter pre-pass launch (the flat
+    layout of a 3-channel input, whose patch-sum kernel carries no filter work, with and without the quad of padding
+    that makes its quad count even; integer-code inputs).  The library's kernel timers then show no launch of
+    px_expand_rows_kernel; every case is checked against the oracle."""
     from tf_approximate_amd import ops
     table = pkg.synth.table_noisy(21)
     ops.set_preexpand(1)
     ops.profile_enable(True)
     try:
-        for xs, fs, strides, own_launch in (((3, 20, 20, 16), (3, 3, 16, 24), (1, 1), False),
-                                            ((2, 30, 30, 64), (1, 1, 64, 40), (1, 1), False),     # flat pixel list
-                                            ((2, 14, 14, 512), (1, 1, 512, 16), (1, 1), False),   # few pixels, many channels
-                                            ((4, 300, 300, 8), (3, 3, 8, 16), (1, 1), False),     # bands of 900 pixels: workgroups
-                                                                                                    # of 1024, a whole fill each
-                                            ((2, 40, 40, 3), (7, 7, 3, 16), (2, 2), True)):
+        for xs, fs, strides, carrier in (((3, 20, 20, 16), (3, 3, 16, 24), (1, 1), "patch_sums"),
+                                         ((2, 30, 30, 64), (1, 1, 64, 40), (1, 1), "patch_sums"),     # flat pixel list
+                                         ((2, 14, 14, 512), (1, 1, 512, 16), (1, 1), "patch_sums"),   # few pixels, many channels
+                                         ((4, 300, 300, 8), (3, 3, 8, 16), (1, 1), "patch_sums"),     # bands of 900 pixels:
+                                                                                                        # workgroups of 1024
+                                         ((2, 40, 40, 3), (7, 7, 3, 16), (2, 2), "filter_pack"),      # 6 quads per filter row
+                                         ((2, 40, 40, 3), (3, 3, 3, 16), (1, 1), "filter_pack")):     # 3 quads and one of padding
             x, f, _, _ = refimpl.grid_case(pkg, xs, fs, MM, seed=sum(xs))
             op = pkg.ApproxConv2DWithMinMaxVars([1, strides[0], strides[1], 1], 8, table, "SAME")
             xd, fd = torch.from_numpy(x).to(gpu_util.dev()), torch.from_numpy(f).to(gpu_util.dev())
@@ -230,11 +232,11 @@ def test_rows_are_built_by_the_pre_pass_launch_where_it_can_carry_them(pkg, orac
             y = op(xd, fd, *MM).cpu().numpy()
             prof = ops.profile_read()
             assert "lutgemm_px" in prof and "lutgemm_expand" not in prof, (xs, prof)
-            assert ("px_expand_rows" in prof) == own_launch, (xs, prof)
+            assert "px_expand_rows" not in prof and ("filter_pack" in prof) == (carrier == "filter_pack"), (xs, prof)
             rc, y_ref, _ = oracle.conv2d_fast(table, x, f, *MM, strides=strides, padding="SAME")
             assert rc == 0
             assert refimpl.linf_rel(y, y_ref) <= 1e-5
-        # the codes entry point: no patch sums, so no launch to ride along with
+        # the codes entry point: no patch sums, the rows ride in the filter pre-pass launch
         xs, fs = (3, 20, 20, 16), (3, 3, 16, 24)
         rng = np.random.default_rng(4)
         qa = rng.integers(0, 256, xs).astype(np.uint8)
@@ -243,7 +245,7 @@ def test_rows_are_built_by_the_pre_pass_launch_where_it_can_carry_them(pkg, orac
         acc = ops.conv2d_codes_acc_i32(pkg.TruthTable(table), torch.from_numpy(qa).to(gpu_util.dev()),
                                        torch.from_numpy(qb).to(gpu_util.dev()), 3, (1, 1, 1, 1), "SAME").cpu().numpy()
         prof = ops.profile_read()
-        assert "lutgemm_px" in prof and "px_expand_rows" in prof, prof
+        assert "lutgemm_px" in prof and "filter_pack" in prof and "px_expand_rows" not in prof, prof
         patches = refimpl.gather_patches(qa, 3, 3, 3, (1, 1), "SAME", (1, 1))
         n, oh, ow = patches.shape[:3]
         want = oracle.lut_gemm_codes(table, patches.reshape(n * oh * ow, -1), qb.reshape(-1, fs[3]))

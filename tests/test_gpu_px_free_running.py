@@ -66,6 +66,8 @@ def test_barrier_free_kernel_whole_output_and_oracle(pkg, oracle, case):
         torch.cuda.synchronize()
         prof = ops.profile_read()
         assert "lutgemm_px" in prof and "lutgemm_expand" not in prof, prof
+        # rows beyond 512 MiB get a launch of their own, the others ride in a pre-pass launch
+        assert ("px_expand_rows" in prof) == (fs[3] * fs[0] * fs[1] * xs[3] * 512 > 512 << 20), prof   # 512 bytes per filter element
         ops.set_preexpand(-1)
         ops.profile_reset()
         y0 = op(xd, fd, *MM)

@@ -523,6 +523,7 @@ DensePlan compute_plan(const ConvGeom &g, int cus, int forced_nt, int px_mode, d
                 }
                 if (cost < best_cost) {
                     best_cost = cost;
+                    best.cost = (float)cost;
                     best.px = px;
                     best.nt = nt;
                     best.rows_per_tile = (int)(wrows * 64);
@@ -662,12 +663,28 @@ int prepare_dense(const axc_conv2d_desc *desc, PreparedDense *pd, bool allow_sub
         const int run = g.KW * g.C, quads = (run + 3) / 4;
         const int64_t row_bytes = std::max<int64_t>((int64_t)(g.pw + g.W) * g.C, (int64_t)(g.OW - 1) * g.sw * g.C + 4 * quads);
         const int64_t rb4 = (row_bytes + 3) & ~(int64_t)3;
-        if (allow_flat && !pd->subsample && (g.C & 3) != 0 && g.dw == 1 && g.pw >= 0 && quads < g.KW * g.C4 &&
-            ((int64_t)g.N * g.H + 2) * rb4 < ((int64_t)1 << 31)) {
+        const bool flat_ok = allow_flat && !pd->subsample && (g.C & 3) != 0 && g.dw == 1 && g.pw >= 0;
+        if (flat_ok && quads < g.KW * g.C4 && ((int64_t)g.N * g.H + 2) * rb4 < ((int64_t)1 << 31)) {
             pd->flat_row_bytes = (int)rb4;
             pd->gk.KW = 1;
             pd->gk.C = run;       // the filter as [KH][KW * C][Co]
             pd->gk.C4 = quads;
+        }
+        // Pre-expanded rows want the quads in pairs.  An odd count (3x3x3: 9 codes, 3 quads, no fewer than the three
+        // one-channel quads of the other layout) may take one more quad, all null weights (its channels lie beyond
+        // KW * C), where the planner then picks those rows and expects the layer to be faster for it.
+        const int64_t row_bytes_p = std::max<int64_t>((int64_t)(g.pw + g.W) * g.C, (int64_t)(g.OW - 1) * g.sw * g.C + 4 * (quads + 1));
+        const int64_t rb4_p = (row_bytes_p + 3) & ~(int64_t)3;
+        if (flat_ok && (quads & 1) && quads >= 3 && ((int64_t)g.N * g.H + 2) * rb4_p < ((int64_t)1 << 31)) {
+            ConvGeom gp = pd->g;
+            gp.KW = 1;
+            gp.C = run;
+            gp.C4 = quads + 1;
+            const DensePlan padded = make_plan(gp, device_cus(), px_mode), plain = make_plan(pd->gk, device_cus(), px_mode);
+            if (padded.px && padded.cost < plain.cost) {
+                pd->gk = gp;
+                pd->flat_row_bytes = (int)rb4_p;
+            }
         }
     }
     pd->plan = make_plan(pd->gk, device_cus(), px_mode);
@@ -802,7 +819,7 @@ int run_dense(const axc_table *table, const axc_conv2d_desc *desc, const float *
     if (!filter_done) {
         ProfScope ps("filter_pack", stream);
         AXC_HIP(launch_filter_pack(codes_mode ? nullptr : filter, filter_codes, gk, pd.plan, tq_f, lq_dev, wq,
-                                   (out_f && !codes_mode) ? fsum : nullptr, stream));
+                                   (out_f && !codes_mode) ? fsum : nullptr, stream, table->dev_tableT, px_rows, &px_done));
     }
 
     DenseParams p;

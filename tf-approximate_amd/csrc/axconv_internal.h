@@ -51,6 +51,7 @@ struct DensePlan {
     int fills_per_split;
     int grid;
     int px;                // 1: the layer suits the kernel that reads pre-expanded rows (lutgemm_px_kernel.hip)
+    float cost;            // what the planner's model expects of the LUT-GEMM launches, in cycles
 };
 
 // Quantization of one tensor as the pre-pass kernels see it.
@@ -228,9 +229,11 @@ hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32
 hipError_t launch_quantize_flat_rows(const float *x, const uint8_t *codes, const ConvGeom &g, int pad_left,
                                      int row_bytes, const TensorQuant &tq, const LayerQuant *lq_dev, uint8_t *xq,
                                      hipStream_t stream);
+// tableT / px_rows / px_done: the launch may also build the pre-expanded rows of the layer (then *px_done is set)
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
                               const DensePlan &plan, const TensorQuant &tq, const LayerQuant *lq_dev,
-                              uint16_t *wq, float *fsum, hipStream_t stream);
+                              uint16_t *wq, float *fsum, hipStream_t stream, const uint16_t *tableT = nullptr,
+                              uint16_t *px_rows = nullptr, bool *px_done = nullptr);
 hipError_t launch_quantize_flat(const float *v, int64_t n, float offset, float inv_scale, uint8_t *codes,
                                 hipStream_t stream);
 hipError_t launch_dense(const DenseParams &p, bool out_i32, hipStream_t stream);

@@ -799,21 +799,53 @@ __device__ __forceinline__ void filter_sums_block(const int block, const float *
 
 // One launch for the whole filter pre-pass: the first sum_blocks workgroups compute the column sums (skipped when
 // fsum is null), the others pack the codes.
+// One (column tile, pair of fills) of the pre-expanded rows (px_expand.h) by a workgroup of 4 * CB threads that is
+// not the one that packs the pair's filter codes: it computes the 128 codes itself, into LDS behind the stage.
+template <int CB>
+__device__ __forceinline__ void px_expand_own_codes(const int eb, const float *__restrict__ filter,
+                                                    const uint8_t *__restrict__ filter_codes, int taps, int C, int C4,
+                                                    int Co, const TensorQuant &q, const uint16_t *__restrict__ tableT,
+                                                    uint16_t *__restrict__ px_rows)
+{
+    extern __shared__ __align__(16) unsigned char px_lds[];
+    uint32_t *const stage = reinterpret_cast<uint32_t *>(px_lds);
+    constexpr int kParts = 256 / CB;
+    const int fills = taps * C4, px_fills = fills / 2;   // 16-column tiles: a fill is one channel quad of a tap
+    const int part = eb % kParts, cf = eb / kParts;      // cf = ct * px_fills + f
+    const int ct = cf / px_fills, f = cf - ct * px_fills;
+    uint16_t *const codes = reinterpret_cast<uint16_t *>(stage + px_expand_stage_dwords<CB>());
+    if (threadIdx.x < 128)
+        codes[threadIdx.x] = filter_code_at(((int64_t)ct * fills + 2 * (int64_t)f) * 64 + threadIdx.x, filter, filter_codes,
+                                            taps, C, C4, Co, 16, q);
+    __syncthreads();
+    px_expand_part<CB>(stage, part, [&](const int sl) { return codes[sl]; }, tableT,
+                       reinterpret_cast<uint32_t *>(px_rows + (size_t)cf * (kPxFillBytes / 2)));
+}
+
+// One launch for the whole filter pre-pass: the first sum_blocks workgroups compute the column sums (skipped when
+// fsum is null), the next pack_blocks pack the codes, any further ones build pre-expanded rows.
 __global__ void __launch_bounds__(kFsThreads) filter_prep_kernel(const float *__restrict__ filter,
                                                                   const uint8_t *__restrict__ filter_codes, int taps,
                                                                   int C, int C4, int Co, int nt, int n_col_tiles,
                                                                   const TensorQuant tq,
                                                                   const LayerQuant *__restrict__ lq_dev,
                                                                   uint16_t *__restrict__ wq, int sum_blocks,
-                                                                  float *__restrict__ fsum)
+                                                                  float *__restrict__ fsum, int pack_blocks,
+                                                                  const uint16_t *__restrict__ tableT,
+                                                                  uint16_t *__restrict__ px_rows)
 {
     const TensorQuant q = lq_dev ? lq_dev->flt : tq;
     if ((int)blockIdx.x < sum_blocks) {
         filter_sums_block<kFsThreads>((int)blockIdx.x, filter, taps * C, Co, q, fsum);
         return;
     }
-    const int64_t i = (int64_t)(blockIdx.x - sum_blocks) * blockDim.x + threadIdx.x;
-    filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, q, wq);
+    const int pb = (int)blockIdx.x - sum_blocks;
+    if (pb < pack_blocks) {
+        const int64_t i = (int64_t)pb * blockDim.x + threadIdx.x;
+        filter_pack_element(i, filter, filter_codes, taps, C, C4, Co, nt, n_col_tiles, q, wq);
+        return;
+    }
+    px_expand_own_codes<kFsThreads / 4>(pb - pack_blocks, filter, filter_codes, taps, C, C4, Co, q, tableT, px_rows);
 }
 
 // Patch sums of a 1x1, stride-1, unpadded layer: the patch of an output pixel is the pixel itself, so the pixels
@@ -1080,29 +1112,12 @@ __device__ __forceinline__ bool filter_work_block(const FilterWork &fw, const La
         filter_pack_element(i, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, fw.nt, fw.n_col_tiles, q, fw.wq);
         return true;
     }
-    // pre-expanded rows (16-column tiles: a fill is one channel quad of a tap, fills = taps x C4): this workgroup
-    // computes the 128 filter codes of its pair of fills into LDS, then expands them
-    extern __shared__ __align__(16) unsigned char px_lds[];
+    // pre-expanded rows: blockDim.x / 4 activation codes of a pair of fills per workgroup
     const int eb = pb - fw.pack_blocks;
-    const int fills = fw.taps * fw.C4, px_fills = fills / 2;
-    uint32_t *const stage = reinterpret_cast<uint32_t *>(px_lds);
-    const auto body = [&](auto cb_tag) {
-        constexpr int CB = decltype(cb_tag)::value;
-        constexpr int kParts = 256 / CB;
-        const int part = eb % kParts, cf = eb / kParts;   // cf = ct * px_fills + f
-        const int ct = cf / px_fills, f = cf - ct * px_fills;
-        uint16_t *const codes = reinterpret_cast<uint16_t *>(stage + px_expand_stage_dwords<CB>());
-        if (threadIdx.x < 128)
-            codes[threadIdx.x] = filter_code_at(((int64_t)ct * fills + 2 * (int64_t)f) * 64 + threadIdx.x, fw.filter,
-                                                fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, 16, q);
-        __syncthreads();
-        px_expand_part<CB>(stage, part, [&](const int sl) { return codes[sl]; }, fw.tableT,
-                           reinterpret_cast<uint32_t *>(fw.px_rows + (size_t)cf * (kPxFillBytes / 2)));
-    };
     if (blockDim.x == 512)
-        body(std::integral_constant<int, 128>());
+        px_expand_own_codes<128>(eb, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, q, fw.tableT, fw.px_rows);
     else
-        body(std::integral_constant<int, 256>());
+        px_expand_own_codes<256>(eb, fw.filter, fw.filter_codes, fw.taps, fw.C, fw.C4, fw.Co, q, fw.tableT, fw.px_rows);
     return true;
 }
 
@@ -1845,19 +1860,33 @@ hipError_t launch_codes_relayout(const uint8_t *codes, const ConvGeom &g, uint32
 
 hipError_t launch_filter_pack(const float *filter, const uint8_t *filter_codes, const ConvGeom &g,
                               const DensePlan &plan, const TensorQuant &tq, const LayerQuant *lq_dev, uint16_t *wq,
-                              float *fsum, hipStream_t stream)
+                              float *fsum, hipStream_t stream, const uint16_t *tableT, uint16_t *px_rows, bool *px_done)
 {
+    if (px_done)
+        *px_done = false;
     const int64_t total = (int64_t)plan.n_col_tiles * plan.fills * 64;
     const int sum_blocks = (fsum && filter) ? (int)blocks_for(g.Co, kFsCols) : 0;
-    const size_t lds = sum_blocks ? kFsLdsBytes : 0;
+    const int pack_blocks = (int)blocks_for(total, kFsThreads);
+    size_t lds = sum_blocks ? kFsLdsBytes : 0;
+    // the pre-expanded rows ride along as in launch_patch_sums: a whole pair of fills per workgroup of 1024
+    int64_t expand_blocks = 0;
+    const size_t row_bytes = (size_t)plan.n_col_tiles * (size_t)(plan.fills / 2) * kPxFillBytes;
+    if (px_done && px_rows && plan.nt == 16 && plan.fills == g.KH * g.KW * g.C4 && (plan.fills & 1) == 0 &&
+        row_bytes <= ((size_t)512 << 20)) {
+        expand_blocks = (int64_t)plan.n_col_tiles * (plan.fills / 2);
+        const size_t need = (size_t)(kFsThreads / 4) * kPxExpandPitch * 4 + 256;
+        lds = lds < need ? need : lds;
+        *px_done = true;
+    }
     if (lds) {
-        const hipError_t ea = set_max_dynamic_lds_once(reinterpret_cast<const void *>(filter_prep_kernel), kFsLdsBytes);
+        const hipError_t ea = set_max_dynamic_lds_once(reinterpret_cast<const void *>(filter_prep_kernel),
+                                                       (int)(lds > (size_t)kFsLdsBytes ? lds : (size_t)kFsLdsBytes));
         if (ea != hipSuccess)
             return ea;
     }
-    hipLaunchKernelGGL(filter_prep_kernel, dim3(sum_blocks + blocks_for(total, kFsThreads)), dim3(kFsThreads), lds,
+    hipLaunchKernelGGL(filter_prep_kernel, dim3((unsigned)(sum_blocks + pack_blocks + expand_blocks)), dim3(kFsThreads), lds,
                        stream, filter, filter_codes, g.KH * g.KW, g.C, g.C4, g.Co, plan.nt, plan.n_col_tiles, tq, lq_dev,
-                       wq, sum_blocks, fsum);
+                       wq, sum_blocks, fsum, pack_blocks, tableT, px_rows);
     return hipGetLastError();
 }
 
