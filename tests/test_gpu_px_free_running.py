@@ -7,7 +7,8 @@ the whole tensor of int32 sums and the whole float output bit for bit against th
 (itself pinned against the oracle by the per-layer tests), sampled pixels against the CPU oracle, and, where torch can
 restate the layer, the whole tensor of sums with the exact table against an fp64 convolution of the codes.  Shapes
 cover even and odd fill counts (a tile that starts in LDS buffer 1), a K split, ragged last row tiles, a column count
-that is no multiple of 16, stride, dilation, the flat 7x7x3 layout, both paddings, and a layer whose pre-expanded rows
+that is no multiple of 16, stride, dilation, the flat 7x7x3 layout, both paddings, tiles of every row count the
+kernel divides differently between its wavefronts, and a layer whose pre-expanded rows
 (1.2 GB) are larger than any cache.  The last test forces the kernel's
 bounded waits to run out and checks the report."""
 import numpy as np
@@ -36,6 +37,16 @@ CASES = [
     ((64, 112, 112, 3), (7, 7, 3, 64), 2, 1, "VALID"),      # flat layout of a 3-channel input, 44-row tiles
     ((32, 28, 28, 512), (3, 3, 512, 512), 1, 1, "SAME"),    # 1.2 GB of rows: read from memory, not from a cache
 ]
+# tiles of 29 to 48 wavefront-rows, which the kernel divides between its older and younger wavefronts by a rule of its
+# own (a second instantiation): 31 rows (20 + 11), 36 (20 + 16), 37 (24 + 13) with a ragged last tile of 19, 47 (28 + 19);
+# the 7x7 stem above has 44 (28 + 16)
+OWN_SPLIT_CASES = [
+    ((64, 31, 64, 16), (3, 3, 16, 64), 1, 1, "SAME"),
+    ((64, 36, 64, 16), (3, 3, 16, 64), 1, 1, "SAME"),
+    ((31, 77, 63, 16), (3, 3, 16, 64), 1, 1, "SAME"),
+    ((64, 47, 64, 16), (3, 3, 16, 64), 1, 1, "SAME"),
+]
+CASES += OWN_SPLIT_CASES
 
 
 def _id(case):
@@ -46,6 +57,11 @@ def _id(case):
 def _plan(pkg, case):
     xs, fs, stride, dil, padding = case
     return pkg.ops.conv2d_tile_plan(xs, fs, (1, stride, stride, 1), padding, (1, dil, dil, 1))
+
+
+def test_own_split_cases_have_such_tiles(pkg):
+    rows = [_plan(pkg, case)["rows_per_tile"] // 64 for case in OWN_SPLIT_CASES]
+    assert rows == [31, 36, 37, 47], rows
 
 
 @pytest.mark.parametrize("case", CASES, ids=_id)

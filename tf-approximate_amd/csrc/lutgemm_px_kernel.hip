@@ -300,7 +300,7 @@ __device__ __forceinline__ void px_count(const uint32_t buffer, const int lane)
 // wavefronts of a SIMD ramp their read windows up and down at different times.  Every wait is a bounded number of
 // polls; a wavefront whose wait runs out raises ABORT, reports through p.wait_error and leaves the kernel, and so do
 // the others when they next wait.
-template <bool OUT_I32>
+template <bool OUT_I32, bool OWN_SPLIT>
 __global__ void __launch_bounds__(kDenseThreads) lutgemm_pxf_kernel(const DenseParams p)
 {
     constexpr int NT = 16, R = 8, PS = 64;   // PS: dwords between a thread's geometry slots (wavefront-major)
@@ -448,7 +448,7 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_pxf_kernel(const DenseP
         const int Ft = F - f0 < Fs ? F - f0 : Fs;
         const uint32_t first_fill = (uint32_t)(ct * F + f0);
         const uint32_t first_fill_next = first_fill_of(ctv_next);
-        const TileRows t = tile_rows_of<R, true, true>(p, rt, wave);
+        const TileRows t = tile_rows_of<R, true, true, OWN_SPLIT>(p, rt, wave);
         const uint32_t nr = park_geometry<R, PS>(p, t, lane, park, skip_row);
         const uint32_t nr_s = __builtin_amdgcn_readfirstlane(nr);
 
@@ -558,10 +558,15 @@ __global__ void __launch_bounds__(kDenseThreads) lutgemm_pxf_kernel(const DenseP
     }
 }
 
-template <bool OUT_I32, bool FREE_RUNNING>
+// FREE_RUNNING: 0 = lutgemm_px_kernel, 1 = lutgemm_pxf_kernel, 2 = lutgemm_pxf_kernel dividing a tile's rows by its
+// own rule (a kernel of its own, so that the other keeps its register allocation: with the rule inside, layers it
+// does not apply to ran 0.3-0.9 % slower)
+template <bool OUT_I32, int FREE_RUNNING>
 static hipError_t launch_px_one(const DenseParams &p, hipStream_t stream)
 {
-    auto kernel = FREE_RUNNING ? lutgemm_pxf_kernel<OUT_I32> : lutgemm_px_kernel<OUT_I32>;
+    auto kernel = FREE_RUNNING == 2   ? lutgemm_pxf_kernel<OUT_I32, true>
+                  : FREE_RUNNING == 1 ? lutgemm_pxf_kernel<OUT_I32, false>
+                                      : lutgemm_px_kernel<OUT_I32>;
     // The generated assembly addresses LDS from offset 0: that holds as long as the kernel has no static LDS in
     // front of its dynamic allocation (checked when the attribute is set, once per device).
     const int lds_bytes = 2 * kPxFillBytes + kDenseParkBytes;
@@ -581,9 +586,14 @@ hipError_t launch_dense_px(const DenseParams &p, bool out_i32, hipStream_t strea
     if (px_free_running(p.plan, p.g.KH * p.g.KW)) {
         if (p.plan.rows_per_tile > 64 * kPxMaxTileWaveRows)   // the control block sits in the last wavefront's last slot
             return hipErrorInvalidValue;
-        return out_i32 ? launch_px_one<true, true>(p, stream) : launch_px_one<false, true>(p, stream);
+        // tiles whose rows tile_rows_of's OWN_SPLIT divides differently: the full ones or the layer's last
+        const int full = p.plan.rows_per_tile / 64;
+        const int last = (int)((p.g.M - (int64_t)(p.plan.n_row_tiles - 1) * p.plan.rows_per_tile + 63) / 64);
+        if ((full >= kOwnSplitFrom && full <= kOwnSplitTo) || (last >= kOwnSplitFrom && last <= kOwnSplitTo))
+            return out_i32 ? launch_px_one<true, 2>(p, stream) : launch_px_one<false, 2>(p, stream);
+        return out_i32 ? launch_px_one<true, 1>(p, stream) : launch_px_one<false, 1>(p, stream);
     }
-    return out_i32 ? launch_px_one<true, false>(p, stream) : launch_px_one<false, false>(p, stream);
+    return out_i32 ? launch_px_one<true, 0>(p, stream) : launch_px_one<false, 0>(p, stream);
 }
 
 // Which of the two kernels a plan with pre-expanded rows runs.  Without barriers the wavefronts of a SIMD drift apart

@@ -22,6 +22,7 @@ __device__ __forceinline__ uint32_t ld_u32(rsrc_t r, uint32_t voff, uint32_t sof
 }
 
 constexpr int kOldShare = 11; // sixteenths of a tile's wavefront-rows owned by the older four wavefronts
+constexpr int kOwnSplitFrom = 29, kOwnSplitTo = 48; // tiles of this many wavefront-rows: tile_rows_of's OWN_SPLIT differs from kOldShare
 
 // The rows of a tile and this wavefront's share of them.  A wavefront-row is 64 consecutive output pixels (one per
 // lane); a wavefront owns wavefront-rows wr_base, wr_base + 4, ... below its half's end.  The SIMD issues the older
@@ -34,7 +35,7 @@ struct TileRows {
 };
 // ROUND_ROBIN: wavefront-row i goes to SIMD i & 3 whichever half owns it (wavefront w sits on SIMD w & 3), so the
 // SIMDs' loads differ by one row at most however the rows divide between the halves.
-template <int R, bool EVEN_SMALL = false, bool ROUND_ROBIN = false>
+template <int R, bool EVEN_SMALL = false, bool ROUND_ROBIN = false, bool OWN_SPLIT = false>
 __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, int wave)
 {
     TileRows t;
@@ -42,6 +43,12 @@ __device__ __forceinline__ TileRows tile_rows_of(const DenseParams &p, int rt, i
     t.row_end = (t.row0 + p.plan.rows_per_tile < p.g.M) ? t.row0 + p.plan.rows_per_tile : p.g.M;
     const int wrows = (int)((t.row_end - t.row0 + 63) / 64);
     int wr_old = (wrows * kOldShare + 8) / 16;
+    // OWN_SPLIT (the kernel without barriers, whose wavefronts are not held to a common pace fill by fill: a tile
+    // takes as long as its longest wavefront).  Measured over tiles of 32-60 wavefront-rows at 72 fills, an older
+    // wavefront with o rows takes 57 + 25.5 o microseconds, a younger one with y rows 13 + 45 y: whole rows per older
+    // wavefront, as many as make the larger of the two smallest.  From 49 rows on that is the rule above.
+    if (OWN_SPLIT && wrows >= kOwnSplitFrom)
+        wr_old = wrows <= 36 ? 20 : wrows <= 40 ? 24 : wrows <= kOwnSplitTo ? 28 : 32;
     // EVEN_SMALL: with up to one wavefront-row per wavefront, one each (for a kernel whose phase then lasts as long
     // as the lookups of its slowest wavefront)
     if (EVEN_SMALL && wrows <= kDenseWaves)
