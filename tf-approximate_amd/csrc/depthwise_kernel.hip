@@ -101,6 +101,19 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut_kernel(const Dept
 // zero-point code) and drop stores, without a branch; columns outside the image are a wave-uniform case.
 // Results are those of depthwise_lut_kernel: taps in (kh, kw) order, the patch sum sequential in that order.
 constexpr int kDwChannels = 32;
+#ifndef AXC_DW_AHEAD
+#define AXC_DW_AHEAD 1
+#endif
+
+// f(integral_constant<int, I>) for I = A .. B-1
+template <int A, int B, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (A < B) {
+        f(std::integral_constant<int, A>());
+        static_for<A + 1, B>(f);
+    }
+}
 constexpr int kDwCodeStride = 5 * kDwChannels * 4;    // bytes between activation codes: five pairs of taps
 constexpr int kDwLdsBytes = 256 * kDwCodeStride;      // 163840
 
@@ -116,7 +129,8 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                                                                           const int group_slots)
 {
     constexpr int RIN = (R - 1) * S + 3;               // input rows under R output rows
-    constexpr int CARRY = 3 - S;                       // window columns the next output column keeps
+    constexpr int AHEAD = AXC_DW_AHEAD;                // output columns by which the loads run ahead of the lookups
+    constexpr int SLOTS = 3 + S * AHEAD;               // window columns held at a time: the 3 in use and those on their way
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -166,12 +180,17 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
         __syncthreads();
 
         const float t3 = (!OUT_I32 && live) ? __fmul_rn(ep.m1, p.fsum[chan]) : 0.0f;
-        const float bias = (!OUT_I32 && p.bias && live) ? p.bias[chan] : 0.0f;
-        const uint32_t lane_off = (uint32_t)cl * 4u;
-        // value -> (fake-quantized value, byte offset of its code's entries)
-        auto convert = [&](float raw, float &val, uint32_t &off) {
-            val = fake_quant_value(raw, q);
-            off = quantize_code(val, q.offset, q.inv_scale) * (uint32_t)kDwCodeStride + lane_off;
+        // bias and ReLU exist at the layer entry point only (FQ).  Without a bias the kernel adds -0.0f, which
+        // changes no value, the sign of a zero included.
+        const bool has_relu = FQ && p.relu;
+        const float bias = (FQ && !OUT_I32 && p.bias && live) ? p.bias[chan] : -0.0f;
+        // LDS address of this lane's entries of activation code 0: the tap is an immediate offset of the read
+        const uint32_t lane_base = (uint32_t)reinterpret_cast<uintptr_t>(lds_dw) + (uint32_t)cl * 4u;
+        typedef const __attribute__((address_space(3))) uint16_t *lds_entry_ptr;
+        // value -> (fake-quantized value, LDS address of its code's entries); the code is below 2^24
+        auto convert = [&](float &val, uint32_t &off) {
+            val = fake_quant_value(val, q);
+            off = __umul24(quantize_code(val, q.offset, q.inv_scale), (uint32_t)kDwCodeStride) + lane_base;
         };
 
         for (int task = run_first + wave; task < run_end; task += kWaves) {
@@ -188,19 +207,6 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                                 ? (uint32_t)((((int64_t)n * p.H + ih) * p.W * p.C + chan) * 4)
                                 : 0x80000000u;
             }
-            // column iw of every window row, or zeros when the column is outside the image (iw is wave-uniform)
-            auto load_col = [&](int iw, float (&dst)[RIN]) {
-                if ((unsigned)iw < (unsigned)p.W) {
-                    const uint32_t coff = (uint32_t)iw * col_bytes;
-#pragma unroll
-                    for (int r = 0; r < RIN; ++r)
-                        dst[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)rowoff[r], (int)coff, 0));
-                } else {
-#pragma unroll
-                    for (int r = 0; r < RIN; ++r)
-                        dst[r] = 0.0f;
-                }
-            };
             uint32_t ooff[R];                           // byte offset of (n, oh0 + rr, 0, chan) in the output
 #pragma unroll
             for (int rr = 0; rr < R; ++rr)
@@ -208,28 +214,48 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                                ? (uint32_t)((((int64_t)(n * p.OH + oh0 + rr) * p.OW) * p.C + chan) * 4)
                                : 0x80000000u;
 
-            float val[RIN][3];
-            uint32_t off[RIN][3];
-            float pf[S][RIN];
-            // window of output column 0: physical slot of window column t at output column k is (S*k + t) % 3
-            {
-                float first[3][RIN];
-#pragma unroll
-                for (int t = 0; t < 3; ++t)
-                    load_col(iw0 + t, first[t]);
-#pragma unroll
-                for (int t = 0; t < 3; ++t)
+            // The window: input column j of the block (j = 0 is column iw0) lives in slot j % SLOTS for as long as an
+            // output column needs it.  SLOTS = 3 + S * AHEAD: the S columns that enter with output column k + AHEAD are
+            // loaded into the slots that column k - 1 left, while column k is computed, and those of column k + 1 are
+            // converted in place afterwards - no value is ever copied from one register to another.  (AHEAD = 2 and 3
+            // measured no faster than 1: the kernel is bound by the memory system, not by a wavefront's latency.)
+            float val[RIN][SLOTS];
+            uint32_t off[RIN][SLOTS];
+            // column iw of every window row into a slot, or zeros when the column is outside the image (iw is
+            // wave-uniform)
+            auto load_col = [&](int iw, auto slot_tag) {
+                constexpr int SL = decltype(slot_tag)::value;
+                if ((unsigned)iw < (unsigned)p.W) {
+                    const uint32_t coff = (uint32_t)iw * col_bytes;
 #pragma unroll
                     for (int r = 0; r < RIN; ++r)
-                        convert(first[t][r], val[r][t], off[r][t]);
-            }
-            auto step = [&](const int k, auto phase_tag) {
-                constexpr int PH = decltype(phase_tag)::value;   // k % 3
-                const bool more = k + 1 < len;
-                if (more) {                                // the columns that enter with output column k + 1
+                        val[r][SL] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)rowoff[r], (int)coff, 0));
+                } else {
 #pragma unroll
-                    for (int s = 0; s < S; ++s)
-                        load_col(iw0 + (k + 1) * S + CARRY + s, pf[s]);
+                    for (int r = 0; r < RIN; ++r)
+                        val[r][SL] = 0.0f;
+                }
+            };
+            auto convert_col = [&](auto slot_tag) {
+                constexpr int SL = decltype(slot_tag)::value;
+#pragma unroll
+                for (int r = 0; r < RIN; ++r)
+                    convert(val[r][SL], off[r][SL]);
+            };
+            // the columns of the first AHEAD output columns
+            static_for<0, 3 + S * (AHEAD - 1)>([&](auto j) { load_col(iw0 + decltype(j)::value, j); });
+            static_for<0, 3>([&](auto j) { convert_col(j); });
+
+            auto step = [&](const int k, auto phase_tag) {
+                constexpr int PH = decltype(phase_tag)::value;   // k % SLOTS
+                // slots of the columns that enter with output column k + AHEAD (loaded now) and with k + 1 (converted
+                // when this column is done)
+                constexpr int LD0 = (S * (PH + AHEAD) + 3 - S) % SLOTS, LD1 = (LD0 + 1) % SLOTS;
+                constexpr int CV0 = (S * PH + 3) % SLOTS, CV1 = (CV0 + 1) % SLOTS;
+                if (k + AHEAD < len) {
+                    load_col(iw0 + (k + AHEAD) * S + 3 - S, std::integral_constant<int, LD0>());
+                    if (S == 2)
+                        load_col(iw0 + (k + AHEAD) * S + 2, std::integral_constant<int, LD1>());
                 }
                 const uint32_t ocol = (uint32_t)(ow0 + k) * col_bytes;
 #pragma unroll
@@ -240,9 +266,10 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                     for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
                         for (int kw = 0; kw < 3; ++kw) {
-                            const int ps = (S * PH + kw) % 3;
+                            const int ps = (S * PH + kw) % SLOTS;
+                            const int tap = kh * 3 + kw;
                             psum = __fadd_rn(psum, val[rr * S + kh][ps]);
-                            e[kh * 3 + kw] = *reinterpret_cast<const uint16_t *>(lds_dw + off[rr * S + kh][ps] + ((kh * 3 + kw) >> 1) * 128 + ((kh * 3 + kw) & 1) * 2);
+                            e[tap] = reinterpret_cast<lds_entry_ptr>(off[rr * S + kh][ps])[(tap >> 1) * 64 + (tap & 1)];
                         }
                     const uint32_t acc = ((e[0] + e[1] + e[2]) + (e[3] + e[4] + e[5])) + (e[6] + e[7] + e[8]);
                     uint32_t outw;
@@ -254,30 +281,24 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                         const float t2 = __fadd_rn(t0, t1);
                         const float t4 = __fadd_rn(t2, t3);
                         float v = __fsub_rn(t4, ep.k_m1xm2);
-                        if (p.bias)
+                        if (FQ)
                             v = __fadd_rn(v, bias);
-                        outw = __float_as_uint(p.relu ? fmaxf(v, 0.0f) : v);
+                        outw = __float_as_uint(has_relu ? fmaxf(v, 0.0f) : v);
                     }
                     // streamed past the caches, which the input rows neighbouring bands share need
                     __builtin_amdgcn_raw_buffer_store_b32(outw, o_rsrc, (int)ooff[rr], (int)ocol, 2);
                 }
-                if (more) {
-#pragma unroll
-                    for (int s = 0; s < S; ++s) {
-                        const int ps = (S * (PH + 1) + CARRY + s) % 3;
-#pragma unroll
-                        for (int r = 0; r < RIN; ++r)
-                            convert(pf[s][r], val[r][ps], off[r][ps]);
-                    }
+                if (k + 1 < len) {
+                    convert_col(std::integral_constant<int, CV0>());
+                    if (S == 2)
+                        convert_col(std::integral_constant<int, CV1>());
                 }
             };
-            for (int k = 0; k < len; k += 3) {
-                step(k, std::integral_constant<int, 0>());
-                if (k + 1 < len)
-                    step(k + 1, std::integral_constant<int, 1>());
-                if (k + 2 < len)
-                    step(k + 2, std::integral_constant<int, 2>());
-            }
+            for (int k = 0; k < len; k += SLOTS)
+                static_for<0, SLOTS>([&](auto ph) {
+                    if (k + decltype(ph)::value < len)
+                        step(k + decltype(ph)::value, ph);
+                });
         }
     }
 }
@@ -310,13 +331,28 @@ hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hi
             group_slots = cus;
         }
         const int band_pairs = (p.OH + 2 * R - 1) / (2 * R);
-        // column segments: enough tasks that every wavefront of a group's workgroups gets several, few window restarts
-        const int64_t waves = (int64_t)wgs_per_group * kWaves;
-        int nseg = 1;
-        while (nseg < p.OW && (int64_t)p.N * band_pairs * nseg < 5 * waves && (p.OW + nseg) / (nseg + 1) >= 8)
-            ++nseg;
-        const int seg_len = (p.OW + nseg - 1) / nseg;
-        nseg = (p.OW + seg_len - 1) / seg_len;
+        // Column segments.  A workgroup deals its run of tasks to its wavefronts in rounds, and a wavefront without a
+        // task in the last round idles while the others work: the number of rounds times the columns a task loads
+        // (its segment and the window's restart) is what a workgroup takes.  The segment count with the smallest such
+        // product among segments of 8 to 24 columns: shorter ones restart the window too often.
+        int nseg = 1, seg_len = p.OW;
+        int64_t best = -1;
+        for (int ns = 1; ns <= p.OW; ++ns) {
+            const int sl = (p.OW + ns - 1) / ns;
+            if (ns > 1 && sl < 8)
+                break;
+            if (sl > 24 && (p.OW + ns) / (ns + 1) >= 8)
+                continue;       // long segments let the wavefronts that share halo rows drift apart (measured: 1 % slower)
+            const int ns_eff = (p.OW + sl - 1) / sl;
+            const int64_t tasks = (int64_t)p.N * band_pairs * ns_eff;
+            const int64_t per_wg = (tasks + wgs_per_group - 1) / wgs_per_group;
+            const int64_t cost = ((per_wg + kWaves - 1) / kWaves) * (sl + 3);
+            if (best < 0 || cost < best) {
+                best = cost;
+                nseg = ns_eff;
+                seg_len = sl;
+            }
+        }
         const int g3 = wgs_per_group * group_slots;
 #define AXC_DW_LAUNCH(S_, R_)                                                                                        \
     (out_i32 ? launch_with_lds(depthwise_lut3x3_kernel<S_, R_, true, false>, g3, kDwLdsBytes, stream, p, seg_len,    \
