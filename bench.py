@@ -82,27 +82,27 @@ CPU_SAMPLE_S = 0.5      # single-thread reference sample per `layers` record
 # device copy of known size inside the same run.  Keyed by (workload, kernel); not measured in the run that prints
 # them: the bench line says which profile they come from.
 PROFILED_TRAFFIC = {
-    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 81249.2 * 1024 + 1.000 * 64118.2 * 1024,
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_px"): (2.000 * 81258.0 * 1024 + 1.000 * 64419.8 * 1024,
                                                            "profiles/lutgemm_px_conv3x3_b64_56x56x64.md"),
-    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8312.5 * 1024 + 1.000 * 60968.5 * 1024,
+    ("conv3x3_b64_56x56x64_to_64_s1_same", "lutgemm_expand"): (2.000 * 8312.5 * 1024 + 1.000 * 61656.5 * 1024,
                                                                "profiles/lutgemm_expand_conv3x3_b64_56x56x64.md"),
-    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48253.9 * 1024 + 1.000 * 790871.3 * 1024,
+    ("conv1x1_b64_112x112x32_to_192", "lutgemm_px"): (2.000 * 48266.1 * 1024 + 1.000 * 792178.1 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b64_112x112x32_to_192.md"),
-    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37308.6 * 1024 + 1.000 * 267897.6 * 1024,
+    ("conv1x1_b64_56x56x64_to_256", "lutgemm_px"): (2.000 * 37216.1 * 1024 + 1.000 * 266473.4 * 1024,
                                                     "profiles/lutgemm_px_conv1x1_b64_56x56x64_to_256.md"),
-    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 471479.0 * 1024 + 1.000 * 470258.6 * 1024,
+    ("conv1x1_b32_56x56x256_to_1024", "lutgemm_px"): (2.000 * 471685.9 * 1024 + 1.000 * 470379.1 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b32_56x56x256_to_1024.md"),
-    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 94017.5 * 1024 + 1.000 * 244842.3 * 1024,
+    ("conv7x7s2_b64_224x224x3_to_64", "lutgemm_px"): (2.000 * 94083.4 * 1024 + 1.000 * 244689.7 * 1024,
                                                       "profiles/lutgemm_px_conv7x7s2_b64_224x224x3_to_64.md"),
-    ("conv3x3_b64_28x28x512_to_512", "lutgemm_px"): (2.000 * 2066521.6 * 1024 + 1.000 * 106139.1 * 1024,
+    ("conv3x3_b64_28x28x512_to_512", "lutgemm_px"): (2.000 * 2065967.7 * 1024 + 1.000 * 106108.0 * 1024,
                                                      "profiles/lutgemm_px_conv3x3_b64_28x28x512_to_512.md"),
-    ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6109.0 * 1024 + 1.025 * 8192.0 * 1024,
+    ("conv3x3_b128_32x32x16_to_16", "lutgemm_px"): (2.050 * 6113.0 * 1024 + 1.025 * 8192.0 * 1024,
                                                     "profiles/lutgemm_px_conv3x3_b128_32x32x16_to_16.md"),
-    ("conv1x1_b64_112x112x192_to_32", "lutgemm_px"): (2.000 * 101813.4 * 1024 + 1.000 * 129997.3 * 1024,
+    ("conv1x1_b64_112x112x192_to_32", "lutgemm_px"): (2.000 * 101823.7 * 1024 + 1.000 * 130117.9 * 1024,
                                                       "profiles/lutgemm_px_conv1x1_b64_112x112x192_to_32.md"),
-    ("conv3x3_b64_28x28x128_to_128", "lutgemm_px"): (2.000 * 130201.6 * 1024 + 1.000 * 54427.9 * 1024,
+    ("conv3x3_b64_28x28x128_to_128", "lutgemm_px"): (2.000 * 130204.7 * 1024 + 1.000 * 54284.1 * 1024,
                                                      "profiles/lutgemm_px_conv3x3_b64_28x28x128_to_128.md"),
-    ("conv3x3_b64_7x7x512_to_512", "lutgemm_expand"): (2.000 * 8854.6 * 1024 + 1.000 * 55287.6 * 1024,
+    ("conv3x3_b64_7x7x512_to_512", "lutgemm_expand"): (2.000 * 8874.8 * 1024 + 1.000 * 55210.4 * 1024,
                                                        "profiles/lutgemm_expand_conv3x3_b64_7x7x512_to_512.md"),
     ("dw3x3_b64_112x112x192_s1", "depthwise_lut"): (2.000 * 362120 * 1024 + 1.000 * 602112 * 1024,
                                                     "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
