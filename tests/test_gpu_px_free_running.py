@@ -38,13 +38,15 @@ CASES = [
     ((32, 28, 28, 512), (3, 3, 512, 512), 1, 1, "SAME"),    # 1.2 GB of rows: read from memory, not from a cache
 ]
 # tiles of 29 to 48 wavefront-rows, which the kernel divides between its older and younger wavefronts by a rule of its
-# own (a second instantiation): 31 rows (20 + 11), 36 (20 + 16), 37 (24 + 13) with a ragged last tile of 19, 47 (28 + 19);
+# own (a second instantiation): 31 rows (20 + 11), 36 (20 + 16; also under a K split), 37 (24 + 13) with a ragged last tile
+# of 19, 47 (28 + 19);
 # the 7x7 stem above has 44 (28 + 16)
 OWN_SPLIT_CASES = [
     ((64, 31, 64, 16), (3, 3, 16, 64), 1, 1, "SAME"),
     ((64, 36, 64, 16), (3, 3, 16, 64), 1, 1, "SAME"),
     ((31, 77, 63, 16), (3, 3, 16, 64), 1, 1, "SAME"),
     ((64, 47, 64, 16), (3, 3, 16, 64), 1, 1, "SAME"),
+    ((64, 36, 64, 64), (3, 3, 64, 16), 1, 1, "SAME"),   # 36-row tiles with K split in four
 ]
 CASES += OWN_SPLIT_CASES
 
@@ -61,7 +63,8 @@ def _plan(pkg, case):
 
 def test_own_split_cases_have_such_tiles(pkg):
     rows = [_plan(pkg, case)["rows_per_tile"] // 64 for case in OWN_SPLIT_CASES]
-    assert rows == [31, 36, 37, 47], rows
+    assert rows == [31, 36, 37, 47, 36], rows
+    assert _plan(pkg, OWN_SPLIT_CASES[4])["k_splits"] == 4
 
 
 @pytest.mark.parametrize("case", CASES, ids=_id)
