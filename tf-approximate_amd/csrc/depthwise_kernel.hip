@@ -221,20 +221,19 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
             // measured no faster than 1: the kernel is bound by the memory system, not by a wavefront's latency.)
             float val[RIN][SLOTS];
             uint32_t off[RIN][SLOTS];
-            // column iw of every window row into a slot, or zeros when the column is outside the image (iw is
-            // wave-uniform)
-            auto load_col = [&](int iw, auto slot_tag) {
+            // Column iw of every window row into a slot; zeros when the column is outside the image or not wanted (both
+            // wave-uniform).  No branch: the offset of such a column is past the end of the buffer, like a row outside
+            // the image.  With a branch around the loads the compiler no longer knows, where the paths meet, which
+            // loads have returned, and waits in every output column for loads - and with them for the stores issued
+            // after them - that have long been waited for.
+            auto load_col = [&](int iw, auto slot_tag, bool wanted) {
                 constexpr int SL = decltype(slot_tag)::value;
-                if ((unsigned)iw < (unsigned)p.W) {
-                    const uint32_t coff = (uint32_t)iw * col_bytes;
+                const bool inside = wanted && (unsigned)iw < (unsigned)p.W;
+                const uint32_t past = inside ? 0u : 0x80000000u;
+                const uint32_t coff = inside ? (uint32_t)iw * col_bytes : 0u;
 #pragma unroll
-                    for (int r = 0; r < RIN; ++r)
-                        val[r][SL] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)rowoff[r], (int)coff, 0));
-                } else {
-#pragma unroll
-                    for (int r = 0; r < RIN; ++r)
-                        val[r][SL] = 0.0f;
-                }
+                for (int r = 0; r < RIN; ++r)
+                    val[r][SL] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(rowoff[r] | past), (int)coff, 0));
             };
             auto convert_col = [&](auto slot_tag) {
                 constexpr int SL = decltype(slot_tag)::value;
@@ -243,7 +242,7 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                     convert(val[r][SL], off[r][SL]);
             };
             // the columns of the first AHEAD output columns
-            static_for<0, 3 + S * (AHEAD - 1)>([&](auto j) { load_col(iw0 + decltype(j)::value, j); });
+            static_for<0, 3 + S * (AHEAD - 1)>([&](auto j) { load_col(iw0 + decltype(j)::value, j, true); });
             static_for<0, 3>([&](auto j) { convert_col(j); });
 
             auto step = [&](const int k, auto phase_tag) {
@@ -252,11 +251,9 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                 // when this column is done)
                 constexpr int LD0 = (S * (PH + AHEAD) + 3 - S) % SLOTS, LD1 = (LD0 + 1) % SLOTS;
                 constexpr int CV0 = (S * PH + 3) % SLOTS, CV1 = (CV0 + 1) % SLOTS;
-                if (k + AHEAD < len) {
-                    load_col(iw0 + (k + AHEAD) * S + 3 - S, std::integral_constant<int, LD0>());
-                    if (S == 2)
-                        load_col(iw0 + (k + AHEAD) * S + 2, std::integral_constant<int, LD1>());
-                }
+                load_col(iw0 + (k + AHEAD) * S + 3 - S, std::integral_constant<int, LD0>(), k + AHEAD < len);
+                if (S == 2)
+                    load_col(iw0 + (k + AHEAD) * S + 2, std::integral_constant<int, LD1>(), k + AHEAD < len);
                 const uint32_t ocol = (uint32_t)(ow0 + k) * col_bytes;
 #pragma unroll
                 for (int rr = 0; rr < R; ++rr) {
@@ -288,11 +285,9 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                     // streamed past the caches, which the input rows neighbouring bands share need
                     __builtin_amdgcn_raw_buffer_store_b32(outw, o_rsrc, (int)ooff[rr], (int)ocol, 2);
                 }
-                if (k + 1 < len) {
-                    convert_col(std::integral_constant<int, CV0>());
-                    if (S == 2)
-                        convert_col(std::integral_constant<int, CV1>());
-                }
+                convert_col(std::integral_constant<int, CV0>());   // behind the last column: zeros, never used
+                if (S == 2)
+                    convert_col(std::integral_constant<int, CV1>());
             };
             for (int k = 0; k < len; k += SLOTS)
                 static_for<0, SLOTS>([&](auto ph) {
