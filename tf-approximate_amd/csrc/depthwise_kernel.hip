@@ -123,7 +123,7 @@ __device__ __forceinline__ dw_rsrc_t dw_make_rsrc(const void *base, uint32_t byt
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
 
-template <int S, int R, bool OUT_I32, bool FQ>
+template <int S, int R, bool OUT_I32, bool FQ, bool EPI>
 __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const DepthwiseParams p, const int seg_len,
                                                                           const int nseg, const int wgs_per_group,
                                                                           const int group_slots)
@@ -180,10 +180,10 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
         __syncthreads();
 
         const float t3 = (!OUT_I32 && live) ? __fmul_rn(ep.m1, p.fsum[chan]) : 0.0f;
-        // bias and ReLU exist at the layer entry point only (FQ).  Without a bias the kernel adds -0.0f, which
-        // changes no value, the sign of a zero included.
-        const bool has_relu = FQ && p.relu;
-        const float bias = (FQ && !OUT_I32 && p.bias && live) ? p.bias[chan] : -0.0f;
+        // EPI: the call has a bias or a ReLU (a template parameter: the plain op pays for neither).  Without a bias
+        // the kernel adds -0.0f, which changes no value, the sign of a zero included.
+        const bool has_relu = EPI && p.relu;
+        const float bias = (EPI && !OUT_I32 && p.bias && live) ? p.bias[chan] : -0.0f;
         // LDS address of this lane's entries of activation code 0: the tap is an immediate offset of the read
         const uint32_t lane_base = (uint32_t)reinterpret_cast<uintptr_t>(lds_dw) + (uint32_t)cl * 4u;
         typedef const __attribute__((address_space(3))) uint16_t *lds_entry_ptr;
@@ -278,7 +278,7 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut3x3_kernel(const D
                         const float t2 = __fadd_rn(t0, t1);
                         const float t4 = __fadd_rn(t2, t3);
                         float v = __fsub_rn(t4, ep.k_m1xm2);
-                        if (FQ)
+                        if (EPI)
                             v = __fadd_rn(v, bias);
                         outw = __float_as_uint(has_relu ? fmaxf(v, 0.0f) : v);
                     }
@@ -349,15 +349,18 @@ hipError_t launch_depthwise(const DepthwiseParams &p, bool out_i32, int grid, hi
             }
         }
         const int g3 = wgs_per_group * group_slots;
+#define AXC_DW_LAUNCH_AS(S_, R_, I32_, FQ_, EPI_)                                                                     \
+    launch_with_lds(depthwise_lut3x3_kernel<S_, R_, I32_, FQ_, EPI_>, g3, kDwLdsBytes, stream, p, seg_len, nseg,         \
+                    wgs_per_group, group_slots)
 #define AXC_DW_LAUNCH(S_, R_)                                                                                        \
-    (out_i32 ? launch_with_lds(depthwise_lut3x3_kernel<S_, R_, true, false>, g3, kDwLdsBytes, stream, p, seg_len,    \
-                               nseg, wgs_per_group, group_slots)                                                     \
-     : p.lq_dev ? launch_with_lds(depthwise_lut3x3_kernel<S_, R_, false, true>, g3, kDwLdsBytes, stream, p, seg_len, \
-                                  nseg, wgs_per_group, group_slots)                                                  \
-                : launch_with_lds(depthwise_lut3x3_kernel<S_, R_, false, false>, g3, kDwLdsBytes, stream, p,         \
-                                  seg_len, nseg, wgs_per_group, group_slots))
+    (out_i32    ? AXC_DW_LAUNCH_AS(S_, R_, true, false, false)                                                           \
+     : p.lq_dev ? AXC_DW_LAUNCH_AS(S_, R_, false, true, true)                                                            \
+     : epi      ? AXC_DW_LAUNCH_AS(S_, R_, false, false, true)                                                           \
+                : AXC_DW_LAUNCH_AS(S_, R_, false, false, false))
+        const bool epi = p.bias != nullptr || p.relu != 0;
         return p.sw == 1 ? AXC_DW_LAUNCH(1, 4) : AXC_DW_LAUNCH(2, 2);
 #undef AXC_DW_LAUNCH
+#undef AXC_DW_LAUNCH_AS
     }
     return out_i32 ? launch_with_lds(depthwise_lut_kernel<true>, grid, kTableBytes, stream, p)
                    : launch_with_lds(depthwise_lut_kernel<false>, grid, kTableBytes, stream, p);
