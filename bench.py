@@ -104,9 +104,9 @@ PROFILED_TRAFFIC = {
                                                      "profiles/lutgemm_px_conv3x3_b64_28x28x128_to_128.md"),
     ("conv3x3_b64_7x7x512_to_512", "lutgemm_expand"): (2.000 * 8874.8 * 1024 + 1.000 * 55210.4 * 1024,
                                                        "profiles/lutgemm_expand_conv3x3_b64_7x7x512_to_512.md"),
-    ("dw3x3_b64_112x112x192_s1", "depthwise_lut"): (2.000 * 362120 * 1024 + 1.000 * 602112 * 1024,
+    ("dw3x3_b64_112x112x192_s1", "depthwise_lut"): (2.000 * 360914 * 1024 + 1.000 * 602112 * 1024,
                                                     "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
-    ("dw3x3_b64_112x112x192_s2", "depthwise_lut"): (2.000 * 314741 * 1024 + 1.000 * 150528 * 1024,
+    ("dw3x3_b64_112x112x192_s2", "depthwise_lut"): (2.000 * 314820 * 1024 + 1.000 * 150528 * 1024,
                                                     "profiles/depthwise_lut3x3_dw3x3_b64_112x112x192.md"),
 }
 
