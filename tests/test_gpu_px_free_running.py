@@ -117,6 +117,49 @@ def test_barrier_free_kernel_whole_output_and_oracle(pkg, oracle, case):
             int(bad.sum()), bad.numel(), tuple(int(v) for v in bad.nonzero()[0]))
 
 
+def _random_layers(pkg, count, seed):
+    """Seeded random layers that the planner gives to the kernel (plan code 2)."""
+    ops = pkg.ops
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        k = int(rng.choice([1, 3, 3, 5]))
+        c = int(rng.choice([16, 24, 32, 48, 64, 96, 128]))
+        co = int(rng.integers(1, 13)) * int(rng.choice([8, 16, 20]))
+        xs = (int(rng.integers(8, 49)), int(rng.integers(20, 70)), int(rng.integers(20, 70)), c)
+        stride, padding = int(rng.choice([1, 1, 2])), str(rng.choice(["SAME", "VALID"]))
+        if xs[0] * xs[1] * xs[2] * max(c, co) > 30e6:
+            continue
+        case = (xs, (k, k, c, co), stride, 1, padding)
+        plan = ops.conv2d_tile_plan(xs, case[1], (1, stride, stride, 1), padding, (1, 1, 1, 1))
+        if plan["preexpanded_rows"] == 2:
+            out.append(case)
+    return out
+
+
+def test_random_full_size_layers_equal_the_expanding_kernel(pkg):
+    """Ninety-six seeded random layers (tile heights, K splits, strides, paddings as the planner makes them): whole sums
+    and whole float outputs bit for bit against the kernel that expands inside its tiles."""
+    ops = pkg.ops
+    heights = set()
+    for i, case in enumerate(_random_layers(pkg, 96, seed=2024)):
+        print("case", _id(case), flush=True)
+        xs, fs, stride, dil, padding = case
+        heights.add(_plan(pkg, case)["rows_per_tile"] // 64)
+        table = pkg.synth.table_random(i)
+        xd, fd = bench.device_tensors(pkg, xs, fs, "uniform", seed=i)
+        op = pkg.ApproxConv2DWithMinMaxVars([1, stride, stride, 1], 8, table, padding)
+        try:
+            acc, y = op.accumulators(xd, fd, *MM), op(xd, fd, *MM)
+            ops.set_preexpand(-1)
+            acc0, y0 = op.accumulators(xd, fd, *MM), op(xd, fd, *MM)
+        finally:
+            ops.set_preexpand(0)
+        assert torch.equal(acc, acc0), _id(case)
+        assert torch.equal(y.view(torch.int32), y0.view(torch.int32)), _id(case)
+    assert len(heights) >= 24, heights
+
+
 def test_dilated_case_against_the_oracle_on_a_crop(pkg, oracle):
     """The dilated case above only compares the two kernels; here the oracle recomputes one whole image of it."""
     xs, fs, stride, dil, padding = CASES[4]
