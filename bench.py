@@ -61,6 +61,8 @@ LAYERS = [
     ("cfg3_inverted_residual", "expand_1x1_32_192", (64, 112, 112, 32), (1, 1, 32, 192), (1, 1), False, "uniform", "trunc2"),
     ("cfg3_inverted_residual", "dw3x3_192_s1", (64, 112, 112, 192), (3, 3, 192, 1), (1, 1), True, "uniform", "trunc4"),
     ("cfg3_inverted_residual", "dw3x3_192_s2", (64, 112, 112, 192), (3, 3, 192, 1), (2, 2), True, "uniform", "trunc2"),
+    # a depthwise filter that is not 3x3 runs the generic kernel (whole table in LDS, one-entry gathers)
+    ("cfg3_inverted_residual", "dw5x5_192_s1_generic", (64, 56, 56, 192), (5, 5, 192, 1), (1, 1), True, "uniform", "trunc4"),
     ("cfg3_inverted_residual", "project_1x1_192_32", (64, 112, 112, 192), (1, 1, 192, 32), (1, 1), False, "uniform", "trunc4"),
     ("cfg4_resnet50", "stem_7x7s2_3_64", (64, 224, 224, 3), (7, 7, 3, 64), (2, 2), False, "uniform", "uniform_error"),
     ("cfg4_resnet50", "stage1_1x1_64_256", (64, 56, 56, 64), (1, 1, 64, 256), (1, 1), False, "uniform", "uniform_error"),
