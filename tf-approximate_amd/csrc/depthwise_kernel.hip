@@ -98,9 +98,10 @@ __global__ void __launch_bounds__(kBlockThreads) depthwise_lut_kernel(const Dept
 // offset once per block instead of once per output row and tap, and rows shared by the R outputs of a column are
 // fetched once.  Both halves of a wavefront walk the same columns, so column offsets are scalars.  Rows outside the
 // image are buffer offsets past the end, which read 0.0f (the value the reference pads with; it quantizes to the
-// zero-point code) and drop stores, without a branch; columns outside the image are a wave-uniform case.
+// zero-point code) and drop stores, without a branch; so are columns outside the image (a wave-uniform case).
 // Results are those of depthwise_lut_kernel: taps in (kh, kw) order, the patch sum sequential in that order.
 constexpr int kDwChannels = 32;
+// output columns by which the window's loads run ahead of its lookups (2 and 3 measured no faster than 1)
 #ifndef AXC_DW_AHEAD
 #define AXC_DW_AHEAD 1
 #endif
